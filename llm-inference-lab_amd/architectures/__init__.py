@@ -1,2 +1,3 @@
 """Architectures known to the framework; importing this package registers them."""
 from . import qwen2  # noqa: F401
+from . import vivevik  # noqa: F401

@@ -53,12 +53,17 @@ def pages_for_tokens(tokens: int, page_size: int) -> int:
     return (tokens + page_size - 1) // page_size
 
 
-def group_page_need(window: Optional[int], page_size: int, total_tokens: int, max_step_tokens: int) -> int:
+def group_page_need(window: Optional[int], page_size: int, total_tokens: int, max_step_tokens: int,
+                    keep_first: int = 0) -> int:
     """Most pages of one group a request holds at any time when it grows to
-    ``total_tokens`` in steps of at most ``max_step_tokens``."""
+    ``total_tokens`` in steps of at most ``max_step_tokens``.  The pages of the first
+    ``keep_first`` positions are held throughout."""
     full = pages_for_tokens(total_tokens, page_size)
     if window is None:
         return full
+    if keep_first:
+        return min(full, pages_for_tokens(keep_first, page_size)
+                   + group_page_need(window, page_size, total_tokens, max_step_tokens))
     # Before a step of n tokens is committed the request holds the pages of the
     # positions [computed - window + 1, computed + n); that span touches at most
     # ceil((window - 1 + n) / P) + 1 pages.
@@ -158,7 +163,7 @@ class CacheManager:
         return [st.get("v") for st in self.storage]
 
     def page_need(self, total_tokens: int, max_step_tokens: int) -> List[int]:
-        return [group_page_need(g.window, self.page_size, total_tokens, max_step_tokens)
+        return [group_page_need(g.window, self.page_size, total_tokens, max_step_tokens, g.spec.keep_first)
                 for g in self.groups]
 
     # -------------------------------------------------------------- lifecycle
@@ -227,7 +232,9 @@ class CacheManager:
             lowest_needed = max(0, req.computed_len - g.window + 1)
             first_needed_page = lowest_needed // self.page_size
             pages = req.pages[gi]
-            for lp in range(req.first_live[gi], min(first_needed_page, len(pages))):
+            # (pages that hold any of the first ``keep_first`` positions stay for good)
+            kept = pages_for_tokens(g.spec.keep_first, self.page_size)
+            for lp in range(max(req.first_live[gi], kept), min(first_needed_page, len(pages))):
                 if pages[lp] != NO_PAGE:
                     self.pools[gi].free(pages[lp], req.row)
                     pages[lp] = NO_PAGE

@@ -58,10 +58,12 @@ def get_architecture(name: str) -> Architecture:
 
 
 def architecture_of(raw: Dict[str, Any], where: str = "config.json") -> Architecture:
-    """The entry that ``architectures[0]`` names.  A configuration without that key (one
+    """The entry that ``architectures[0]`` (or the single name ``architecture``) names.  A configuration without that key (one
     written by hand for the random-weights mode) is matched by its ``model_type`` against
     the ``MODEL_TYPE`` of the registered configuration classes."""
     archs = raw.get("architectures")
+    if archs is None and isinstance(raw.get("architecture"), str):       # (one name, not a list)
+        return get_architecture(raw["architecture"])
     if archs is None and isinstance(raw.get("model_type"), str):
         hits = [a for a in _ARCHITECTURES.values()
                 if getattr(a.config_class, "MODEL_TYPE", None) == raw["model_type"]]

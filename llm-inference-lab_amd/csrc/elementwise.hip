@@ -4,7 +4,7 @@
 
 extern "C" const char* llmlab_last_error() { return g_llmlab_error; }
 
-extern "C" int llmlab_abi_version() { return 6; }
+extern "C" int llmlab_abi_version() { return 7; }
 
 // --------------------------------------------------------------- embedding
 // out[r, :] = float(table[ids[r], :]); an id outside [0, vocab) is clamped (the
@@ -484,5 +484,104 @@ extern "C" int llmlab_add_pending(float* x, const float* pend, int splits, size_
   hipLaunchKernelGGL(add_pending_kernel, dim3((unsigned)((count + 255) / 256)), dim3(256), 0, stream, x, pend,
                      splits, stride, count);
   LLMLAB_LAUNCH_CHECK("add_pending");
+  return 0;
+}
+
+// ------------------------------------------------------------- layer norm
+// y = (x - mean(x)) * rsqrt(var(x) + eps) * w with var the mean of the squared
+// deviations (taken about the mean, in a pass of its own), no bias; all in float32.
+// ADD false: out[i, :] = T(y) for x row rows[i] (or i).  ADD true: the float32 stream
+// resid[i, :] += y, and, if copy is given, copy[i, :] = T(resid[i, :]) after the sum: what
+// the next reader of the stream multiplies with.
+template <typename T, bool ADD>
+__global__ __launch_bounds__(256) void layernorm_kernel(const float* __restrict__ x, const void* __restrict__ w,
+                                                        int w_bf16, float eps, T* __restrict__ out,
+                                                        float* __restrict__ resid, T* __restrict__ copy,
+                                                        const int* __restrict__ rows, int hidden) {
+  __shared__ float red[17];
+  const int i = blockIdx.x;
+  const float* src = x + (size_t)(rows ? rows[i] : i) * hidden;
+  float s = 0.f;
+  for (int c = threadIdx.x; c < hidden; c += blockDim.x) s += src[c];
+  const float mean = block_sum(s, red) / (float)hidden;
+  float v = 0.f;
+  for (int c = threadIdx.x; c < hidden; c += blockDim.x) {
+    const float d = src[c] - mean;
+    v += d * d;
+  }
+  const float inv = 1.0f / sqrtf(block_sum(v, red) / (float)hidden + eps);
+  for (int c = threadIdx.x; c < hidden; c += blockDim.x) {
+    const float y = (src[c] - mean) * inv * load_vec(w, w_bf16, c);
+    if (ADD) {
+      const float t = resid[(size_t)i * hidden + c] + y;
+      resid[(size_t)i * hidden + c] = t;
+      if (copy) copy[(size_t)i * hidden + c] = from_float<T>(t);
+    } else {
+      out[(size_t)i * hidden + c] = from_float<T>(y);
+    }
+  }
+}
+
+// out: n_out rows of the compute dtype; rows: which rows of x (null: all in order).
+extern "C" int llmlab_layernorm(const float* x, const void* w, int w_dtype, float eps, void* out, int out_dtype,
+                                const int* rows, int n_out, int hidden, hipStream_t stream) {
+  LLMLAB_REQUIRE(n_out >= 0 && hidden > 0, "layernorm: bad sizes n=%d hidden=%d", n_out, hidden);
+  if (n_out == 0) return 0;
+  if (out_dtype == DT_BF16)
+    hipLaunchKernelGGL((layernorm_kernel<bf16_t, false>), dim3(n_out), dim3(256), 0, stream, x, w, w_dtype == DT_BF16,
+                       eps, (bf16_t*)out, (float*)nullptr, (bf16_t*)nullptr, rows, hidden);
+  else
+    hipLaunchKernelGGL((layernorm_kernel<float, false>), dim3(n_out), dim3(256), 0, stream, x, w, w_dtype == DT_BF16,
+                       eps, (float*)out, (float*)nullptr, (float*)nullptr, rows, hidden);
+  LLMLAB_LAUNCH_CHECK("layernorm");
+  return 0;
+}
+
+// resid += layernorm(y); copy (may be null, of copy_dtype) receives the new rows of resid.
+extern "C" int llmlab_layernorm_add(const float* y, const void* w, int w_dtype, float eps, float* resid, void* copy,
+                                    int copy_dtype, int n_rows, int hidden, hipStream_t stream) {
+  LLMLAB_REQUIRE(n_rows >= 0 && hidden > 0, "layernorm_add: bad sizes n=%d hidden=%d", n_rows, hidden);
+  LLMLAB_REQUIRE(y != resid, "layernorm_add: the sublayer's output and the stream are two buffers");
+  if (n_rows == 0) return 0;
+  if (copy_dtype == DT_BF16)
+    hipLaunchKernelGGL((layernorm_kernel<bf16_t, true>), dim3(n_rows), dim3(256), 0, stream, y, w, w_dtype == DT_BF16,
+                       eps, (bf16_t*)nullptr, resid, (bf16_t*)copy, (const int*)nullptr, hidden);
+  else
+    hipLaunchKernelGGL((layernorm_kernel<float, true>), dim3(n_rows), dim3(256), 0, stream, y, w, w_dtype == DT_BF16,
+                       eps, (float*)nullptr, resid, (float*)copy, (const int*)nullptr, hidden);
+  LLMLAB_LAUNCH_CHECK("layernorm_add");
+  return 0;
+}
+
+// ------------------------------------------------- activations on float32 sums
+#define ACT_CAST 0        // out = T(x)
+#define ACT_RELU2 1       // out = T(max(x, 0)^2)
+#define ACT_ZERO 2        // out = 0
+template <typename T, int ACT>
+__global__ void activation_kernel(const float* __restrict__ x, T* __restrict__ out, size_t n) {
+  for (size_t i = (size_t)blockIdx.x * blockDim.x + threadIdx.x; i < n; i += (size_t)gridDim.x * blockDim.x) {
+    float v = ACT == ACT_ZERO ? 0.f : x[i];
+    if (ACT == ACT_RELU2) {
+      v = fmaxf(v, 0.f);
+      v = v * v;
+    }
+    out[i] = from_float<T>(v);
+  }
+}
+
+// The float32 output of a product becomes the next product's input (compute dtype) through
+// an activation.  In float32 ``out`` may be ``x`` itself.
+extern "C" int llmlab_activation(const float* x, void* out, int out_dtype, int act, long n, hipStream_t stream) {
+  LLMLAB_REQUIRE(n >= 0 && act >= ACT_CAST && act <= ACT_ZERO, "activation: bad arguments n=%ld act=%d", n, act);
+  if (n == 0) return 0;
+  const int blocks = (int)((n + 255) / 256 < 65535 ? (n + 255) / 256 : 65535);
+#define LLMLAB_ACT(T, A) hipLaunchKernelGGL((activation_kernel<T, A>), dim3(blocks), dim3(256), 0, stream, x, (T*)out, (size_t)n)
+  if (out_dtype == DT_BF16) {
+    if (act == ACT_RELU2) LLMLAB_ACT(bf16_t, ACT_RELU2); else if (act == ACT_ZERO) LLMLAB_ACT(bf16_t, ACT_ZERO); else LLMLAB_ACT(bf16_t, ACT_CAST);
+  } else {
+    if (act == ACT_RELU2) LLMLAB_ACT(float, ACT_RELU2); else if (act == ACT_ZERO) LLMLAB_ACT(float, ACT_ZERO); else LLMLAB_ACT(float, ACT_CAST);
+  }
+#undef LLMLAB_ACT
+  LLMLAB_LAUNCH_CHECK("activation");
   return 0;
 }

@@ -133,11 +133,25 @@ class CausalLM:
         groups: List[GroupLayout] = []
         by_spec: Dict[object, int] = {}
         state_specs: Dict[int, dict] = {}
-        for view, entry in zip(self.entries, self.spec.schedule):
-            mixer = self.blocks[entry.block].mixer_part()
+        mixers = [self.blocks[entry.block].mixer_part() for entry in self.spec.schedule]
+        # A run that reads another run's cache may do so through a window of its own: the
+        # owner's pages are kept for as long as any of its readers looks back.
+        needs = {i: m.cache_spec() for i, m in enumerate(mixers)
+                 if self.spec.schedule[i].cache_of is None and m.cache_spec() is not None}
+        for i, entry in enumerate(self.spec.schedule):
+            need = mixers[i].cache_spec()
+            if entry.cache_of is not None and need is not None:
+                owner_need = needs.get(entry.cache_of)
+                if owner_need is None or owner_need.tensors != need.tensors:
+                    raise ValueError(
+                        f"schedule[{i}] reads the cache of schedule[{entry.cache_of}], "
+                        f"which keeps {owner_need.tensors if owner_need else None}, not its own {need.tensors}")
+                needs[entry.cache_of] = owner_need.widened_by(need)
+        for view, entry, mixer in zip(self.entries, self.spec.schedule, mixers):
             need = mixer.cache_spec()
             if need is not None:
                 if entry.cache_of is None:
+                    need = needs[view.index]
                     if need not in by_spec:
                         by_spec[need] = len(groups)
                         groups.append(GroupLayout(need, []))
@@ -147,11 +161,6 @@ class CausalLM:
                     groups[view.group].entries.append(view.index)
                 else:
                     owner = self.entries[entry.cache_of]
-                    owner_need = self.blocks[self.spec.schedule[entry.cache_of].block].mixer_part().cache_spec()
-                    if owner_need != need:
-                        raise ValueError(
-                            f"schedule[{view.index}] reads the cache of schedule[{entry.cache_of}], "
-                            f"whose need {owner_need} differs from its own {need}")
                     view.group, view.slot, view.writes_cache = owner.group, owner.slot, False
             elif entry.cache_of is not None:
                 raise ValueError(f"schedule[{view.index}] names a cache but its mixer keeps none")

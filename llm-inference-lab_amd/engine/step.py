@@ -123,6 +123,7 @@ class StepContext:
         # (the whole arrays behind ``q_start`` and ``start_pos``, for a caller that checks once
         # what it will use for steps of any number of requests)
         self.all_q_start, self.all_start_pos = self._view("q_start", b + 1), self._view("start_pos", b)
+        self.all_req_rows = self._view("req_rows", b)
         self._set_views()
 
     def _view(self, name: str, count: int) -> torch.Tensor:
@@ -355,7 +356,7 @@ class StepFunction:
                 continue
             for b in range(ctx.n_reqs):
                 seen = ctx.host_start_pos[b] + ctx.host_q_start[b + 1] - ctx.host_q_start[b]
-                total += per_token * min(seen, g.window)
+                total += per_token * min(seen, g.window + g.spec.keep_first)
         return total
 
     def _decode_auto(self) -> torch.Tensor:

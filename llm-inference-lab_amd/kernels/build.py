@@ -1,8 +1,9 @@
 """Builds the HIP libraries for gfx950 with hipcc and finds built ones.
 
-Two kinds of library: ``core`` (embedding, norm, rotary + cache write, matrix
-products, sampling) and ``attn_d<D>`` (attention for head size D; one per head
-size that a model needs); beside them ``measure`` (stream and matrix-instruction loops for
+Kinds of library: ``core`` (embedding, norms, rotary + cache write, matrix
+products, sampling), ``attn_d<D>`` (attention for head size D; one per head
+size that a model needs), ``windowed_attention`` and ``linear_attention`` (mixers whose
+sizes are run-time arguments; built when a model names them); beside them ``measure`` (stream and matrix-instruction loops for
 the benchmark's measured peaks) and the plain C++ references of the same operations,
 built with the host compiler for the tests.  A library's file name carries a hash of its sources
 and flags, so a library built from other sources is never loaded.  Libraries are
@@ -140,6 +141,16 @@ def attention_library(head_dim: int, force: bool = False) -> str:
     return _compile(f"attn_d{head_dim}", (ATTENTION_SOURCE,), (f"-DHEAD_DIM={head_dim}",), force)
 
 
+# Mixers with run-time sizes: one library each, whatever the head sizes of the model.
+MIXER_SOURCES = {"windowed_attention": "windowed_attention.hip", "linear_attention": "linear_attention.hip"}
+
+
+def mixer_library(kind: str, force: bool = False) -> str:
+    """``windowed_attention``: sliding window with a kept prefix and a sink term;
+    ``linear_attention``: the gated recurrence with a matrix state per head."""
+    return _compile(kind, (MIXER_SOURCES[kind],), (), force)
+
+
 MEASURE_SOURCE = "measure.hip"
 
 
@@ -187,11 +198,13 @@ def reference_library(force: bool = False) -> str:
 
 def library(kind: str, parameter=None, force: bool = False) -> str:
     """The library a part names in ``kernel_libraries()``: ``("core", None)`` or
-    ``("attention", head_dim)``."""
+    ``("attention", head_dim)``, ``("windowed_attention", None)``, ``("linear_attention", None)``."""
     if kind == "core":
         return core_library(force)
     if kind == "attention":
         return attention_library(int(parameter), force)
+    if kind in MIXER_SOURCES:
+        return mixer_library(kind, force)
     raise ValueError(f"no kernel library of kind '{kind}'")
 
 
@@ -200,6 +213,8 @@ def build_all(head_dims: Sequence[int] = DEFAULT_HEAD_DIMS, force: bool = True) 
     out = {"core": core_library(force)}
     for d in head_dims:
         out[f"attn_d{d}"] = attention_library(d, force)
+    for kind in MIXER_SOURCES:
+        out[kind] = mixer_library(kind, force)
     out["measure"] = measure_library(force)
     out["reference"] = reference_library(force)
     return out

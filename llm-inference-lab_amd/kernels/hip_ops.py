@@ -142,9 +142,10 @@ class HipOps:
             self.device = torch.device("cuda", torch.cuda.current_device())
         self._core = self._load(build.core_library())
         self._declare_core()
-        if self._core.llmlab_abi_version() != 6:
+        if self._core.llmlab_abi_version() != 7:
             raise RuntimeError("kernel library and Python bindings disagree on the interface")
         self._attn: Dict[int, ctypes.CDLL] = {}
+        self._mixer_libs: Dict[str, ctypes.CDLL] = {}
         self._shared: Dict[int, tuple] = {}
         self.num_cus = int(torch.cuda.get_device_properties(self.device).multi_processor_count)
         self.workspace = torch.empty(self.WORKSPACE_FLOATS, dtype=torch.float32, device=self.device)
@@ -211,6 +212,13 @@ class HipOps:
             _c_ptr, _c_int, _c_int, _c_size, _c_int, _c_size, _c_ptr]
         c.llmlab_add_pending.argtypes = [_c_ptr, _c_ptr, _c_int, _c_size, _c_int, _c_int, _c_ptr]
         c.llmlab_add_pending.restype = _c_int
+        c.llmlab_layernorm.argtypes = [_c_ptr, _c_ptr, _c_int, _c_float, _c_ptr, _c_int, _c_ptr, _c_int, _c_int, _c_ptr]
+        c.llmlab_layernorm.restype = _c_int
+        c.llmlab_layernorm_add.argtypes = [_c_ptr, _c_ptr, _c_int, _c_float, _c_ptr, _c_ptr, _c_int, _c_int, _c_int,
+                                           _c_ptr]
+        c.llmlab_layernorm_add.restype = _c_int
+        c.llmlab_activation.argtypes = [_c_ptr, _c_ptr, _c_int, _c_int, _c_long, _c_ptr]
+        c.llmlab_activation.restype = _c_int
         for fn in (c.llmlab_embed, c.llmlab_rmsnorm, c.llmlab_rope_kv_write, c.llmlab_rope_inplace,
                    c.llmlab_linear, c.llmlab_sample, c.llmlab_skinny_linear,
                    c.llmlab_linear_partials, c.llmlab_linear_qkv):
@@ -917,6 +925,244 @@ class HipOps:
         return AttentionCall(self, lib, args, most_requests=min(q_start.numel() - 1, start_pos.numel(), block_table.shape[0]),
                              most_context=block_table.shape[1] * page_size, row_req=self._ptr(row_req),
                              heads=(num_heads, num_kv_heads), dtype=qkv.dtype)
+
+    # ------------------------------------------- layer norm, plain activations
+    def layernorm(self, x, weight, eps, out, rows=None) -> None:
+        """``out[i] = (x[r] - mean) / sqrt(var + eps) * weight`` for ``r = rows[i]`` (all rows in
+        order when ``rows`` is None); ``x`` float32, ``out`` the compute dtype."""
+        self._need(x, "norm input", torch.float32)
+        self._need(weight, "norm weight")
+        self._need(out, "norm output")
+        hidden, n_out = x.shape[1], out.shape[0]
+        if weight.numel() != hidden or out.shape[1] != hidden:
+            raise ValueError(f"layernorm: x {tuple(x.shape)}, weight {tuple(weight.shape)}, out {tuple(out.shape)} do not fit")
+        if rows is None:
+            if n_out != x.shape[0]:
+                raise ValueError("layernorm: output rows differ from input rows")
+        else:
+            self._need(rows, "norm row indices", torch.int32)
+            if rows.numel() != n_out:
+                raise ValueError("layernorm: one row index per output row")
+        self._call(self._core.llmlab_layernorm, self._ptr(x), self._ptr(weight), _dt(weight), float(eps),
+                   self._ptr(out), _dt(out), self._ptr(rows), n_out, hidden, self._stream())
+
+    def layernorm_add(self, y, weight, eps, resid, copy=None) -> None:
+        """``resid += layernorm(y)`` on the float32 stream; ``copy`` (compute dtype, same shape)
+        receives the stream's new rows for the product that reads them next."""
+        self._need(y, "sublayer output", torch.float32)
+        self._need(resid, "residual stream", torch.float32)
+        self._need(weight, "norm weight")
+        rows, hidden = resid.shape
+        if tuple(y.shape) != (rows, hidden) or weight.numel() != hidden or y.data_ptr() == resid.data_ptr():
+            raise ValueError(f"layernorm_add: y {tuple(y.shape)}, weight {tuple(weight.shape)}, stream "
+                             f"{tuple(resid.shape)} do not fit (and are two buffers)")
+        if copy is not None:
+            self._need(copy, "copy of the stream")
+            if tuple(copy.shape) != (rows, hidden):
+                raise ValueError("layernorm_add: the copy has the stream's shape")
+        self._call(self._core.llmlab_layernorm_add, self._ptr(y), self._ptr(weight), _dt(weight), float(eps),
+                   self._ptr(resid), self._ptr(copy), _dt(copy) if copy is not None else DT_F32, rows, hidden,
+                   self._stream())
+
+    ACTIVATIONS = {"cast": 0, "relu2": 1, "zero": 2}
+
+    def activation(self, x, out, kind: str) -> None:
+        """``out = act(x)`` element by element, ``x`` float32, ``out`` any kernel dtype of the same
+        shape (``cast``: the value itself; ``relu2``: ``max(x, 0) ** 2``; ``zero``: 0 whatever ``x``)."""
+        self._need(x, "activation input", torch.float32)
+        self._need(out, "activation output")
+        if kind not in self.ACTIVATIONS:
+            raise ValueError(f"unknown activation '{kind}'; known: {', '.join(sorted(self.ACTIVATIONS))}")
+        if tuple(x.shape) != tuple(out.shape):
+            raise ValueError(f"activation: {tuple(x.shape)} -> {tuple(out.shape)}")
+        self._call(self._core.llmlab_activation, self._ptr(x), self._ptr(out), _dt(out), self.ACTIVATIONS[kind],
+                   x.numel(), self._stream())
+
+    # --------------------------------- mixers with run-time sizes (own libraries)
+    def _mixer_lib(self, kind: str) -> ctypes.CDLL:
+        lib = self._mixer_libs.get(kind)
+        if lib is None:
+            lib = self._load(build.mixer_library(kind))
+            lib.llmlab_last_error.restype = ctypes.c_char_p
+            if kind == "windowed_attention":
+                lib.llmlab_project_norm_write.argtypes = [
+                    _c_ptr, _c_int, _c_int, _c_int, _c_int, _c_int, _c_int, _c_int, _c_int, _c_float, _c_ptr, _c_ptr,
+                    _c_ptr, _c_ptr, _c_ptr, _c_int, _c_int, _c_ptr, _c_ptr, _c_ptr, _c_int, _c_ptr]
+                lib.llmlab_project_norm_write.restype = _c_int
+                lib.llmlab_sink_window_attention.argtypes = [
+                    _c_ptr, _c_int, _c_int, _c_int, _c_int, _c_int, _c_int, _c_ptr, _c_ptr, _c_ptr, _c_int, _c_int,
+                    _c_ptr, _c_ptr, _c_int, _c_int, _c_ptr, _c_float, _c_ptr, _c_ptr]
+                lib.llmlab_sink_window_attention.restype = _c_int
+            elif kind == "linear_attention":
+                lib.llmlab_gla_decay.argtypes = [_c_ptr, _c_int, _c_int, _c_int, _c_ptr, _c_ptr, _c_float, _c_ptr,
+                                                 _c_int, _c_ptr]
+                lib.llmlab_gla_decay.restype = _c_int
+                lib.llmlab_gla_slices.argtypes = [_c_int]
+                lib.llmlab_gla_slices.restype = _c_int
+                lib.llmlab_gla_scan.argtypes = [_c_ptr, _c_int, _c_int, _c_int, _c_int, _c_ptr, _c_float, _c_int, _c_int,
+                                                _c_int, _c_ptr, _c_ptr, _c_ptr, _c_int, _c_ptr, _c_ptr]
+                lib.llmlab_gla_scan.restype = _c_int
+                lib.llmlab_gla_output.argtypes = [_c_ptr, _c_int, _c_int, _c_int, _c_int, _c_ptr, _c_float, _c_ptr,
+                                                  _c_int, _c_int, _c_ptr, _c_int, _c_ptr]
+                lib.llmlab_gla_output.restype = _c_int
+            self._mixer_libs[kind] = lib
+            self.loaded_libraries.append(lib._name)
+        return lib
+
+    def check_windowed_attention_sizes(self, num_heads, num_kv_heads, key_dim, value_dim, dtype) -> None:
+        if num_heads % num_kv_heads:
+            raise UnsupportedSizeError(f"{num_heads} heads are not a multiple of {num_kv_heads} kv heads")
+        if not 0 < value_dim <= 256 or not 0 < key_dim <= 4096:
+            raise UnsupportedSizeError(f"windowed attention takes keys up to 4096 and values up to 256 wide, "
+                                       f"got {key_dim} and {value_dim}")
+        self._mixer_lib("windowed_attention")
+
+    def check_linear_attention_sizes(self, num_heads, key_dim, value_dim) -> None:
+        if not 0 < key_dim <= 16 * 1024 or not 0 < value_dim <= 1024:
+            raise UnsupportedSizeError(f"the linear attention scan takes up to 16384 key channels and 1024 value "
+                                       f"channels per head, got {key_dim} and {value_dim}")
+        self._mixer_lib("linear_attention")
+
+    def _paged(self, k_cache, v_cache, num_kv_heads, page_size, key_dim, value_dim, dtype):
+        pages = k_cache.shape[0]
+        if (tuple(k_cache.shape) != (pages, num_kv_heads, page_size, key_dim)
+                or tuple(v_cache.shape) != (pages, num_kv_heads, page_size, value_dim)
+                or not k_cache.is_contiguous() or not v_cache.is_contiguous()):
+            raise ValueError("windowed attention: cache tensors are pages [pages, kv heads, P, width]")
+        if k_cache.dtype != dtype or v_cache.dtype != dtype:
+            raise TypeError("windowed attention: queries and cache share one dtype")
+
+    def project_norm_write(self, proj, num_heads, num_kv_heads, key_dim, value_dim, own_kv, q_norm, k_norm, eps,
+                           q_out, k_cache, v_cache, page_size, positions, row_req, block_table) -> None:
+        """From the float32 projections ``proj [rows, >= q (+ k + v)]``: the queries (divided by
+        the root mean square over their whole width and multiplied by ``q_norm`` if that is
+        given) into ``q_out``, and, if the layer has keys and values of its own, the keys
+        (normed alike with ``k_norm``) and values into the rows' places in the pages."""
+        lib = self._mixer_lib("windowed_attention")
+        self._need(proj, "projections", torch.float32)
+        self._need(q_out, "queries")
+        rows = q_out.shape[0]
+        q_size = num_heads * key_dim
+        need = q_size + (num_kv_heads * (key_dim + value_dim) if own_kv else 0)
+        if proj.shape[0] != rows or proj.shape[1] < need or tuple(q_out.shape) != (rows, q_size):
+            raise ValueError(f"project_norm_write: projections {tuple(proj.shape)}, queries {tuple(q_out.shape)} "
+                             f"do not fit {need} numbers a row")
+        norm = q_norm is not None
+        if norm:
+            self._need(q_norm, "query norm weight", torch.float32)
+            if q_norm.numel() != q_size:
+                raise ValueError("project_norm_write: the query norm's weight spans all heads")
+        if own_kv:
+            self._paged(k_cache, v_cache, num_kv_heads, page_size, key_dim, value_dim, q_out.dtype)
+            if norm:
+                self._need(k_norm, "key norm weight", torch.float32)
+                if k_norm.numel() != num_kv_heads * key_dim:
+                    raise ValueError("project_norm_write: the key norm's weight spans all kv heads")
+            for t, name in ((positions, "positions"), (row_req, "row -> request map"), (block_table, "block table")):
+                self._need(t, name, torch.int32, contiguous=name != "block table")
+            if positions.numel() < rows or row_req.numel() < rows or block_table.stride(1) != 1:
+                raise ValueError("project_norm_write: one position and one request index per row")
+        self._call(lib.llmlab_project_norm_write, self._ptr(proj), proj.stride(0), rows, num_heads, num_kv_heads,
+                   key_dim, value_dim, 1 if own_kv else 0, 1 if norm else 0, float(eps), self._ptr(q_norm),
+                   self._ptr(k_norm) if own_kv and norm else None, self._ptr(q_out),
+                   self._ptr(k_cache) if own_kv else None, self._ptr(v_cache) if own_kv else None, _dt(q_out),
+                   page_size, self._ptr(positions) if own_kv else None, self._ptr(row_req) if own_kv else None,
+                   self._ptr(block_table) if own_kv else None, block_table.stride(0) if own_kv else 0,
+                   self._stream(), lib=lib)
+
+    def sink_window_attention(self, q, num_heads, num_kv_heads, key_dim, value_dim, k_cache, v_cache, block_table,
+                              page_size, positions, row_req, window, keep_first, sink, scale, out) -> None:
+        """The query of row ``r`` at position ``i = positions[r]`` of request ``row_req[r]`` attends
+        to the cached keys ``j <= i`` with ``i - j < window`` or ``j < keep_first`` (``window`` None:
+        all); ``sink`` (float32 per head, or None) adds ``exp(sink)`` to the softmax's denominator."""
+        lib = self._mixer_lib("windowed_attention")
+        self._need(q, "queries")
+        self._need(out, "attention output")
+        rows = q.shape[0]
+        if tuple(q.shape) != (rows, num_heads * key_dim) or tuple(out.shape) != (rows, num_heads * value_dim):
+            raise ValueError(f"windowed attention: queries {tuple(q.shape)}, output {tuple(out.shape)} do not fit "
+                             f"{num_heads} heads of {key_dim} / {value_dim}")
+        if q.dtype != out.dtype:
+            raise TypeError("windowed attention: queries and output share one dtype")
+        self._paged(k_cache, v_cache, num_kv_heads, page_size, key_dim, value_dim, q.dtype)
+        for t, name in ((positions, "positions"), (row_req, "row -> request map")):
+            self._need(t, name, torch.int32)
+            if t.numel() < rows:
+                raise ValueError(f"windowed attention: one entry of {name} per row")
+        self._need(block_table, "block table", torch.int32, contiguous=False)
+        if block_table.stride(1) != 1:
+            raise ValueError("windowed attention: block table rows are contiguous")
+        if sink is not None:
+            self._need(sink, "sink", torch.float32)
+            if sink.numel() != num_heads:
+                raise ValueError("windowed attention: one sink per head")
+        if value_dim > 256:
+            raise UnsupportedSizeError(f"windowed attention takes values up to 256 wide, got {value_dim}")
+        self._call(lib.llmlab_sink_window_attention, self._ptr(q), _dt(q), rows, num_heads, num_kv_heads, key_dim,
+                   value_dim, self._ptr(k_cache), self._ptr(v_cache), self._ptr(block_table), block_table.stride(0),
+                   page_size, self._ptr(positions), self._ptr(row_req), int(window) if window else 0,
+                   int(keep_first or 0), self._ptr(sink), float(scale), self._ptr(out), self._stream(), lib=lib)
+
+    def gla_slices(self, key_dim: int) -> int:
+        """Into how many pieces the scan leaves each output (one per slice of key channels)."""
+        return int(self._mixer_lib("linear_attention").llmlab_gla_slices(int(key_dim)))
+
+    def gla_decay(self, low, rank, w2, bias, tau, decay) -> None:
+        """``decay[r, c] = sigmoid(bias[c] + w2[c] . low[r, :rank]) ** (1 / tau)``, all float32."""
+        lib = self._mixer_lib("linear_attention")
+        for t, name in ((low, "low-rank projection"), (w2, "decay weight"), (decay, "decays")):
+            self._need(t, name, torch.float32, contiguous=name != "low-rank projection")
+        rows, channels = decay.shape
+        if low.shape[0] != rows or low.shape[1] < rank or low.stride(1) != 1 or tuple(w2.shape) != (channels, rank):
+            raise ValueError(f"gla_decay: low {tuple(low.shape)}, weight {tuple(w2.shape)}, decays "
+                             f"{tuple(decay.shape)} do not fit rank {rank}")
+        if bias is not None:
+            self._need(bias, "decay bias", torch.float32)
+            if bias.numel() != channels:
+                raise ValueError("gla_decay: one bias per channel")
+        self._call(lib.llmlab_gla_decay, self._ptr(low), low.stride(0), rows, int(rank), self._ptr(w2),
+                   self._ptr(bias), float(tau), self._ptr(decay), channels, self._stream(), lib=lib)
+
+    def gla_scan(self, proj, off_q, off_k, off_v, decay, q_scale, num_heads, key_dim, value_dim, state, q_start,
+                 req_rows, n_reqs, parts) -> None:
+        """The recurrence ``S = decay_t * S + k_t v_t^T; o_t = S^T (q_scale q_t)`` over the rows
+        ``q_start[b] .. q_start[b + 1]`` of each of the step's ``n_reqs`` requests, on the float32
+        state ``state[req_rows[b]]`` ``[heads, key_dim, value_dim]``, which is left updated;
+        ``parts [rows, heads, gla_slices(key_dim), value_dim]`` receives each output in pieces."""
+        lib = self._mixer_lib("linear_attention")
+        for t, name in ((proj, "projections"), (decay, "decays"), (state, "recurrent state"), (parts, "output pieces")):
+            self._need(t, name, torch.float32)
+        self._need(q_start, "request row starts", torch.int32)
+        self._need(req_rows, "state slots", torch.int32)
+        rows = proj.shape[0]
+        slices = self.gla_slices(key_dim)
+        if (tuple(decay.shape) != (rows, num_heads * key_dim)
+                or tuple(parts.shape) != (rows, num_heads, slices, value_dim)
+                or tuple(state.shape[1:]) != (num_heads, key_dim, value_dim)
+                or q_start.numel() < n_reqs + 1 or req_rows.numel() < n_reqs
+                or min(off_q, off_k, off_v) < 0
+                or max(off_q + num_heads * key_dim, off_k + num_heads * key_dim, off_v + num_heads * value_dim) > proj.shape[1]):
+            raise ValueError("gla_scan: the operands do not fit each other")
+        self._call(lib.llmlab_gla_scan, self._ptr(proj), proj.stride(0), int(off_q), int(off_k), int(off_v),
+                   self._ptr(decay), float(q_scale), num_heads, key_dim, value_dim, self._ptr(state),
+                   self._ptr(q_start), self._ptr(req_rows), int(n_reqs), self._ptr(parts), self._stream(), lib=lib)
+
+    def gla_output(self, parts, num_heads, key_dim, value_dim, weight, eps, proj, off_gate, out) -> None:
+        """``out[r, h] = rmsnorm(sum of parts[r, h]) * weight * silu(gate[r, h])`` with the gate at
+        column ``off_gate`` of the float32 ``proj``; ``out`` in the compute dtype."""
+        lib = self._mixer_lib("linear_attention")
+        self._need(parts, "output pieces", torch.float32)
+        self._need(proj, "projections", torch.float32)
+        self._need(weight, "output norm weight", torch.float32)
+        self._need(out, "mixer output")
+        rows = parts.shape[0]
+        if (tuple(parts.shape) != (rows, num_heads, self.gla_slices(key_dim), value_dim) or weight.numel() != value_dim
+                or tuple(out.shape) != (rows, num_heads * value_dim) or proj.shape[0] != rows
+                or off_gate < 0 or off_gate + num_heads * value_dim > proj.shape[1]):
+            raise ValueError("gla_output: the operands do not fit each other")
+        self._call(lib.llmlab_gla_output, self._ptr(parts), rows, num_heads, key_dim, value_dim, self._ptr(weight),
+                   float(eps), self._ptr(proj), proj.stride(0), int(off_gate), self._ptr(out), _dt(out),
+                   self._stream(), lib=lib)
 
     # --------------------------------------------------------------- sampling
     def argmax(self, logits, out, one_pass: bool = True) -> None:

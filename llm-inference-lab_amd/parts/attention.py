@@ -7,8 +7,8 @@ from typing import Dict, Optional
 import torch
 
 from ..config.spec import PartSpec
-from ..weights.loader import TensorSpec, MATRIX, VECTOR
-from .base import Mixer, KVCacheSpec, NormedInput
+from ..weights.loader import TensorSpec, MATRIX, VECTOR, INIT_NORM
+from .base import Mixer, KVCacheSpec, CacheSpec, PageTensor, NormedInput, PendingSums
 from .registry import register_part, build_part
 
 
@@ -217,4 +217,135 @@ class GQAAttention(Mixer):
         return total
 
 
+class WindowedSinkAttention(Mixer):
+    """Grouped-query attention through a sliding window that keeps a sequence's first
+    positions in sight, with a learned extra term in the softmax's denominator.
+
+    ``q = Wq h`` (``heads x key_dim``), ``k = Wk h`` (``kv_heads x key_dim``), ``v = Wv h``
+    (``kv_heads x value_dim``), no biases.  ``qk_norm="whole"``: q, and k alike, is divided by
+    the root mean square over its WHOLE width (all heads at once, ``eps`` inside the root)
+    and multiplied by a weight of that width, in float32, before it is cut into heads.  The
+    query at position i sees key j if ``j <= i and (i - j < window or j < keep_first)``
+    (``window`` None: every ``j <= i``).  Scores ``q.k * scale``; weights ``exp(s_j - m) /
+    (sum_j exp(s_j - m) + exp(sink_h - m))`` where ``sink_h`` is one learned number per head
+    (``sink=False``: the plain softmax): the extra term has no key and no value.  Head ``h``
+    reads kv head ``h // (heads / kv_heads)``.  No position encoding enters the scores.
+
+    ``own_kv=False``: the layer has no key and value projections; its run reads the pages
+    of the run that the schedule names as its cache (keys as that run stored them, after
+    its norm), with its own queries, window and sink.
+
+    Pages: keys ``[kv_heads, P, key_dim]``, values ``[kv_heads, P, value_dim]``."""
+
+    writes_output = True
+
+    def __init__(self, hidden_size: int, num_heads: int, num_kv_heads: int, key_dim: int, value_dim: int,
+                 scale: float, tensors: Dict[str, str], window: Optional[int] = None, keep_first: int = 0,
+                 sink: bool = True, qk_norm: Optional[str] = "whole", norm_eps: float = 1e-6,
+                 own_kv: bool = True):
+        super().__init__(tensors)
+        if num_heads % num_kv_heads:
+            raise ValueError(f"{num_heads} heads are not a multiple of {num_kv_heads} kv heads")
+        if qk_norm not in (None, "whole"):
+            raise ValueError(f"qk_norm is None or 'whole', got {qk_norm!r}")
+        self.hidden_size, self.num_heads, self.num_kv_heads = int(hidden_size), int(num_heads), int(num_kv_heads)
+        self.key_dim, self.value_dim = int(key_dim), int(value_dim)
+        self.scale = float(scale)
+        self.window = None if window is None else int(window)
+        self.keep_first = int(keep_first or 0)
+        self.has_sink, self.qk_norm, self.norm_eps, self.own_kv = bool(sink), qk_norm, float(norm_eps), bool(own_kv)
+        self.w_in = self.w_o = self.q_norm = self.k_norm = self.sink = None
+
+    @property
+    def q_size(self):
+        return self.num_heads * self.key_dim
+
+    @property
+    def k_size(self):
+        return self.num_kv_heads * self.key_dim
+
+    @property
+    def v_size(self):
+        return self.num_kv_heads * self.value_dim
+
+    @property
+    def in_size(self):
+        return self.q_size + (self.k_size + self.v_size if self.own_kv else 0)
+
+    def tensor_specs(self):
+        t, w = self.tensor_names, self.hidden_size
+        specs = {t["q_weight"]: TensorSpec((self.q_size, w), MATRIX),
+                 t["o_weight"]: TensorSpec((w, self.num_heads * self.value_dim), MATRIX)}
+        if self.own_kv:
+            specs[t["k_weight"]] = TensorSpec((self.k_size, w), MATRIX)
+            specs[t["v_weight"]] = TensorSpec((self.v_size, w), MATRIX)
+        if self.qk_norm:
+            specs[t["q_norm"]] = TensorSpec((self.q_size,), VECTOR, INIT_NORM)
+            if self.own_kv:
+                specs[t["k_norm"]] = TensorSpec((self.k_size,), VECTOR, INIT_NORM)
+        if self.has_sink:
+            specs[t["sink"]] = TensorSpec((self.num_heads,), VECTOR)
+        return specs
+
+    def bind(self, tensors, ops, dtype):
+        super().bind(tensors, ops, dtype)
+        ops.check_windowed_attention_sizes(self.num_heads, self.num_kv_heads, self.key_dim, self.value_dim, dtype)
+        ops.check_product_sizes(self.hidden_size, dtype, "attention projections (hidden size)")
+        ops.check_product_sizes(self.num_heads * self.value_dim, dtype, "attention output projection (heads * value size)")
+        t = self.tensor_names
+        rows = [tensors[t["q_weight"]]]
+        if self.own_kv:
+            rows += [tensors[t["k_weight"]], tensors[t["v_weight"]]]
+        self.w_in = ops.prepare_weight(torch.cat(rows, dim=0).contiguous())       # one product for q (, k, v)
+        self.w_o = ops.prepare_weight(tensors[t["o_weight"]].contiguous())
+        if self.qk_norm:
+            self.q_norm = tensors[t["q_norm"]].float().contiguous()
+            self.k_norm = tensors[t["k_norm"]].float().contiguous() if self.own_kv else None
+        if self.has_sink:
+            self.sink = tensors[t["sink"]].float().contiguous()
+
+    def cache_spec(self):
+        return CacheSpec((("k", PageTensor((self.num_kv_heads, self.key_dim), 1)),
+                          ("v", PageTensor((self.num_kv_heads, self.value_dim), 1))),
+                         self.window, self.keep_first if self.window is not None else 0)
+
+    def forward_into(self, h, out, ctx, entry):
+        ops, rows = self.ops, h.shape[0]
+        if self.own_kv != bool(entry.writes_cache):
+            raise ValueError("an attention layer without keys and values of its own reads another run's cache, "
+                             "and one that has them writes its own")
+        group = ctx.group(entry.group)
+        proj = ctx.scratch("windowed_attention.proj", (rows, self.in_size), torch.float32)
+        ops.linear_logits(h, self.w_in, proj)
+        q = ctx.scratch("windowed_attention.q", (rows, self.q_size), self.dtype)
+        ops.project_norm_write(proj, self.num_heads, self.num_kv_heads, self.key_dim, self.value_dim, self.own_kv,
+                               self.q_norm, self.k_norm, self.norm_eps, q, entry.k_cache, entry.v_cache,
+                               group.page_size, ctx.positions, ctx.row_req, group.block_table)
+        mixed = ctx.scratch("windowed_attention.out", (rows, self.num_heads * self.value_dim), self.dtype)
+        ops.sink_window_attention(q, self.num_heads, self.num_kv_heads, self.key_dim, self.value_dim, entry.k_cache,
+                                  entry.v_cache, group.block_table, group.page_size, ctx.positions, ctx.row_req,
+                                  self.window, self.keep_first, self.sink, self.scale, mixed)
+        ops.linear_logits(mixed, self.w_o, out)
+
+    def forward(self, h, residual, ctx, entry):
+        if isinstance(h, NormedInput):
+            h = h.tensor()
+        y = ctx.scratch("windowed_attention.sum", (1,) + tuple(residual.shape), torch.float32)
+        self.forward_into(h, y[0], ctx, entry)
+        self.ops.add_pending(residual, PendingSums(y, 1))
+
+    keeps_launches = True      # (every argument is a buffer of the step or a size of the layer)
+
+    def kernel_libraries(self):
+        return [("windowed_attention", None)]
+
+    def weight_bytes(self):
+        total = 0
+        for w in (self.w_in, self.w_o, self.q_norm, self.k_norm, self.sink):
+            if w is not None:
+                total += w.numel() * w.element_size()
+        return total
+
+
 register_part("mixer", "gqa_attention", GQAAttention)
+register_part("mixer", "windowed_sink_attention", WindowedSinkAttention)

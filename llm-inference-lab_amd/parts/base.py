@@ -50,12 +50,15 @@ class PageTensor:
 class CacheSpec:
     """What a mixer keeps for each token: named tensors in pages.  ``window``: how many
     of the latest positions (the current one included) it ever reads, or ``None`` for
-    all.  Mixers with equal specs share one group of pages and one block table; the cache
+    all; ``keep_first``: how many of a sequence's first positions it goes on reading after
+    the window has passed them (their pages are never given back while the request lives).
+    Mixers with equal specs share one group of pages and one block table; the cache
     manager allocates ``[runs, pages, *page_shape]`` per name and a run of the mixer finds
     its slices in ``entry.cache[name]``."""
 
     tensors: Tuple[Tuple[str, PageTensor], ...]
     window: Optional[int] = None
+    keep_first: int = 0
 
     def __post_init__(self):
         names = [n for n, _ in self.tensors]
@@ -63,6 +66,14 @@ class CacheSpec:
             raise ValueError(f"a cache spec names at least one tensor, each once: {names}")
         if self.window is not None and self.window <= 0:
             raise ValueError(f"a window holds at least the current position, got {self.window}")
+        if self.keep_first < 0:
+            raise ValueError(f"keep_first counts positions, got {self.keep_first}")
+
+    def widened_by(self, other: "CacheSpec") -> "CacheSpec":
+        """The same tensors kept long enough for ``other``'s reads as well (a run that reads
+        another run's cache through a window of its own)."""
+        window = None if self.window is None or other.window is None else max(self.window, other.window)
+        return dataclasses.replace(self, window=window, keep_first=max(self.keep_first, other.keep_first))
 
     def bytes_per_token(self, dtype: torch.dtype) -> int:
         return sum(t.token_elements() * torch.empty((), dtype=t.dtype or dtype).element_size()
@@ -215,6 +226,11 @@ class PositionEncoding(Part):
 
 class Mixer(Part):
     takes_normed_input = False     # True: ``forward`` gets a ``NormedInput`` and may fuse the norm
+    # True: the part also has ``forward_into(h, out, ctx, ...)``, which WRITES its result into
+    # the float32 ``out`` instead of adding it into the stream (for blocks that put a norm
+    # between the sublayer and the sum).  Without it such a block hands ``forward`` a zeroed
+    # buffer in place of the stream.
+    writes_output = False
 
     def cache_spec(self) -> Optional[CacheSpec]:
         """Per-token cache need (``KVCacheSpec(...)`` for keys and values, or any
@@ -235,6 +251,7 @@ class Mixer(Part):
 
 class FeedForward(Part):
     takes_normed_input = False
+    writes_output = False          # as for mixers: ``forward_into(h, out, ctx)``
 
     def forward(self, h: torch.Tensor, residual: torch.Tensor, ctx) -> None:
         """``residual += feed_forward(h)``."""

@@ -55,6 +55,88 @@ class PreNormBlock(Block):
         return sum(p.weight_bytes() for p in self.parts())
 
 
+class SublayerNormBlock(Block):
+    """``x += norm1(mixer(x)); x += norm2(feed_forward(x))``: the sublayers read the stream
+    itself and each norm acts on its sublayer's OUTPUT, before the sum.  A block without a
+    feed-forward has the first half only.  The stream and both sums are float32; the
+    sublayers' products read the stream rounded to the compute dtype.
+
+    A part that ``writes_output`` writes its float32 result into a scratch buffer
+    (``forward_into``); any other part (made for blocks that add the sublayer's result
+    straight into the stream) is handed a zeroed buffer in the stream's place."""
+
+    def __init__(self, hidden_size: int, mixer: PartSpec, norm1: PartSpec, feed_forward: PartSpec = None,
+                 norm2: PartSpec = None, tensors: Dict[str, str] = None):
+        super().__init__(tensors)
+        if (feed_forward is None) != (norm2 is None):
+            raise ValueError("a feed-forward and its norm come together")
+        self.hidden_size = int(hidden_size)
+        self.mixer = build_part("mixer", mixer)
+        self.norm1 = build_part("norm", norm1)
+        self.feed_forward = build_part("feed_forward", feed_forward) if feed_forward is not None else None
+        self.norm2 = build_part("norm", norm2) if norm2 is not None else None
+        for n in (self.norm1, self.norm2):
+            if n is not None and not hasattr(n, "add_into"):
+                raise ValueError(f"{type(n).__name__} cannot norm a sublayer's output into the stream (no add_into)")
+
+    def parts(self):
+        return [p for p in (self.mixer, self.norm1, self.feed_forward, self.norm2) if p is not None]
+
+    def mixer_part(self):
+        return self.mixer
+
+    def tensor_specs(self):
+        specs = {}
+        for p in self.parts():
+            specs.update(p.tensor_specs())
+        return specs
+
+    def bind(self, tensors, ops, dtype):
+        super().bind(tensors, ops, dtype)
+        for p in self.parts():
+            p.bind(tensors, ops, dtype)
+
+    def _fold(self, residual, ctx):
+        pending = getattr(ctx, "pending", None)
+        if pending is not None:          # (sums another kind of block left in pieces)
+            self.ops.add_pending(residual, pending)
+            ctx.pending = None
+
+    def _input(self, residual, ctx):
+        """The stream as the sublayers' products read it."""
+        if self.dtype == torch.float32:
+            return residual
+        h = ctx.scratch("block.stream_copy", tuple(residual.shape), self.dtype)
+        self.ops.activation(residual, h, "cast")
+        return h
+
+    def _sublayer(self, part, h, residual, ctx, *entry):
+        y = ctx.scratch("block.sublayer_out", tuple(residual.shape), torch.float32)
+        if part.writes_output:
+            part.forward_into(h, y, ctx, *entry)
+        else:
+            self.ops.activation(y, y, "zero")
+            part.forward(h, y, ctx, *entry)
+            self._fold(y, ctx)
+        return y
+
+    def forward(self, residual, ctx, entry):
+        self._fold(residual, ctx)
+        h = self._input(residual, ctx)
+        y = self._sublayer(self.mixer, h, residual, ctx, entry)
+        if self.feed_forward is None:
+            self.norm1.add_into(y, residual)
+            return
+        # the sum's new rows go to the feed-forward in the same pass
+        copy = h if self.dtype != torch.float32 else None
+        self.norm1.add_into(y, residual, copy)
+        y = self._sublayer(self.feed_forward, h, residual, ctx)
+        self.norm2.add_into(y, residual)
+
+    def weight_bytes(self):
+        return sum(p.weight_bytes() for p in self.parts())
+
+
 class TokenEmbedding(Part):
     """``x[r] = table[id_r]`` into the float32 residual stream
     (rust/engine/src/runner/model/qwen2/kernels.rs:46-57)."""
@@ -121,5 +203,6 @@ class LinearHead(Part):
 
 
 register_part("block", "prenorm", PreNormBlock)
+register_part("block", "sublayer_norm", SublayerNormBlock)
 register_part("embedding", "token_embedding", TokenEmbedding)
 register_part("head", "linear_head", LinearHead)

@@ -92,4 +92,57 @@ class SwiGLU(FeedForward):
         return sum(w.numel() * w.element_size() for w in (self.w_gate_up, self.w_down))
 
 
+class DenseFeedForward(FeedForward):
+    """``W_down act(W_up h)`` with no gate and no biases; ``activation="relu2"``: ``act(z) =
+    max(z, 0) ** 2``, taken on the float32 sums of the first product and rounded once."""
+
+    writes_output = True
+    keeps_launches = True
+    ACTIVATIONS = ("relu2",)
+
+    def __init__(self, hidden_size: int, intermediate_size: int, tensors: Dict[str, str],
+                 activation: str = "relu2"):
+        super().__init__(tensors)
+        if activation not in self.ACTIVATIONS:
+            raise ValueError(f"a dense feed-forward takes the activations {self.ACTIVATIONS}, got '{activation}'")
+        self.hidden_size, self.intermediate_size = int(hidden_size), int(intermediate_size)
+        self.activation = activation
+        self.w_up = self.w_down = None
+
+    def tensor_specs(self):
+        t, h, i = self.tensor_names, self.hidden_size, self.intermediate_size
+        return {t["up_weight"]: TensorSpec((i, h), MATRIX), t["down_weight"]: TensorSpec((h, i), MATRIX)}
+
+    def bind(self, tensors, ops, dtype):
+        super().bind(tensors, ops, dtype)
+        ops.check_product_sizes(self.hidden_size, dtype, "feed-forward (hidden size)")
+        ops.check_product_sizes(self.intermediate_size, dtype, "feed-forward (intermediate size)")
+        t = self.tensor_names
+        self.w_up = ops.prepare_weight(tensors[t["up_weight"]].contiguous())
+        self.w_down = ops.prepare_weight(tensors[t["down_weight"]].contiguous())
+
+    def _activated(self, h, ctx):
+        rows = h.shape[0]
+        sums = ctx.scratch("dense_ffn.sums", (rows, self.intermediate_size), torch.float32)
+        self.ops.linear_logits(h, self.w_up, sums)
+        if self.dtype == torch.float32:
+            act = sums
+        else:
+            act = ctx.scratch("dense_ffn.act", (rows, self.intermediate_size), self.dtype)
+        self.ops.activation(sums, act, self.activation)
+        return act
+
+    def forward_into(self, h, out, ctx):
+        self.ops.linear_logits(self._activated(h, ctx), self.w_down, out)
+
+    def forward(self, h, residual, ctx):
+        if isinstance(h, NormedInput):
+            h = h.tensor()
+        self.ops.linear_residual(self._activated(h, ctx), self.w_down, residual, None)
+
+    def weight_bytes(self):
+        return sum(w.numel() * w.element_size() for w in (self.w_up, self.w_down))
+
+
 register_part("feed_forward", "swiglu", SwiGLU)
+register_part("feed_forward", "dense", DenseFeedForward)

@@ -47,4 +47,36 @@ class RMSNorm(Norm):
         return self.weight.numel() * self.weight.element_size()
 
 
+class LayerNorm(Norm):
+    """``y = (x - mean(x)) / sqrt(var(x) + eps) * w`` with ``var`` the mean of the squared
+    deviations, a weight and no bias; everything in float32, one rounding at the end.
+    ``add_into`` serves blocks that norm a sublayer's OUTPUT: ``stream += norm(y)``."""
+
+    keeps_launches = True
+
+    def __init__(self, size: int, eps: float, tensors: Dict[str, str]):
+        super().__init__(tensors)
+        self.size = int(size)
+        self.eps = float(eps)
+        self.weight: Optional[torch.Tensor] = None
+
+    def tensor_specs(self):
+        return {self.tensor_names["weight"]: TensorSpec((self.size,), VECTOR, INIT_NORM)}
+
+    def bind(self, tensors, ops, dtype):
+        super().bind(tensors, ops, dtype)
+        self.weight = tensors[self.tensor_names["weight"]].contiguous()
+
+    def forward(self, x, out, rows=None):
+        self.ops.layernorm(x, self.weight, self.eps, out, rows)
+
+    def add_into(self, y, stream, copy=None):
+        """``stream += norm(y)``; ``copy`` (compute dtype) receives the stream's new rows."""
+        self.ops.layernorm_add(y, self.weight, self.eps, stream, copy)
+
+    def weight_bytes(self):
+        return self.weight.numel() * self.weight.element_size()
+
+
 register_part("norm", "rmsnorm", RMSNorm)
+register_part("norm", "layernorm", LayerNorm)

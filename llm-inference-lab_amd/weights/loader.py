@@ -42,7 +42,9 @@ INIT_ONES = "ones"
 class TensorSpec:
     """What a part expects of a tensor of the model file: its shape, how it is kept
     (``kind``), and how the random-weights mode draws it (``init``).  The part that owns
-    the tensor says all three; nothing is read off the tensor's name."""
+    the tensor says all three; nothing is read off the tensor's name.  A size of ``None`` in
+    ``shape`` is one that the model file decides: any length is taken there, and the part
+    reads it off the tensor it is bound to."""
 
     shape: Tuple[int, ...]
     kind: str = MATRIX
@@ -71,7 +73,7 @@ def check_names_and_shapes(expected: Dict[str, TensorSpec], found: Dict[str, Tup
         if name not in found:
             continue
         shape, dtype = found[name]
-        if tuple(shape) != tuple(spec.shape):
+        if len(shape) != len(spec.shape) or any(e is not None and int(e) != int(f) for e, f in zip(spec.shape, shape)):
             wrong_shape.append((name, tuple(spec.shape), tuple(shape)))
         is_int = dtype in (torch.int64, torch.int32, torch.int16, torch.int8, torch.uint8, torch.bool)
         if is_int != (spec.kind == INT_TABLE):

@@ -58,7 +58,8 @@ class EmuOps:
     RECORDED = ("embed", "gather_tokens", "rmsnorm", "linear", "linear_residual", "linear_partials",
                 "add_pending", "linear_logits", "linear_swiglu", "fused_norm_qkv", "qkv_rope_cache",
                 "fused_norm_swiglu", "fused_norm_logits", "rope_inplace", "rope_kv_write",
-                "paged_attention", "argmax", "sample")
+                "paged_attention", "argmax", "sample", "layernorm", "layernorm_add", "activation",
+                "project_norm_write", "sink_window_attention", "gla_decay", "gla_scan", "gla_output")
 
     def __init__(self, device="cpu", fuse=True):
         self.device = torch.device(device)
@@ -222,6 +223,113 @@ class EmuOps:
         gate = y[:, :, 0, :].reshape(x.shape[0], -1)[:, :inter]
         up = y[:, :, 1, :].reshape(x.shape[0], -1)[:, :inter]
         out.copy_((gate / (1.0 + torch.exp(-gate)) * up).to(out.dtype))
+
+    # ------------------------------------------- layer norm, plain activations
+    @staticmethod
+    def _layernorm(v, weight, eps):
+        mean = v.mean(-1, keepdim=True)
+        var = ((v - mean) ** 2).mean(-1, keepdim=True)
+        return (v - mean) / torch.sqrt(var + eps) * weight.float()
+
+    def layernorm(self, x, weight, eps, out, rows=None):
+        self._count("layernorm")
+        v = x.float() if rows is None else x.float()[rows.long()]
+        out.copy_(self._layernorm(v, weight, eps).to(out.dtype))
+
+    def layernorm_add(self, y, weight, eps, resid, copy=None):
+        self._count("layernorm_add")
+        resid.add_(self._layernorm(y.float(), weight, eps))
+        if copy is not None:
+            copy.copy_(resid.to(copy.dtype))
+
+    def activation(self, x, out, kind):
+        self._count("activation")
+        v = x.float()
+        v = {"cast": v, "relu2": torch.relu(v) ** 2, "zero": torch.zeros_like(v)}[kind]
+        out.copy_(v.to(out.dtype))
+
+    # --------------------------------- mixers with run-time sizes
+    def check_windowed_attention_sizes(self, num_heads, num_kv_heads, key_dim, value_dim, dtype):
+        pass
+
+    def check_linear_attention_sizes(self, num_heads, key_dim, value_dim):
+        pass
+
+    def project_norm_write(self, proj, num_heads, num_kv_heads, key_dim, value_dim, own_kv, q_norm, k_norm, eps,
+                           q_out, k_cache, v_cache, page_size, positions, row_req, block_table):
+        self._count("project_norm_write")
+        rows = q_out.shape[0]
+        qs, ks, vs = num_heads * key_dim, num_kv_heads * key_dim, num_kv_heads * value_dim
+
+        def whole(v, w):
+            return v if w is None else v / torch.sqrt((v * v).mean(-1, keepdim=True) + eps) * w.float()
+        p = proj.float()
+        q_out.copy_(whole(p[:, :qs], q_norm).to(q_out.dtype))
+        if not own_kv:
+            return
+        k = whole(p[:, qs:qs + ks], k_norm).to(k_cache.dtype).view(rows, num_kv_heads, key_dim)
+        v = p[:, qs + ks:qs + ks + vs].to(v_cache.dtype).view(rows, num_kv_heads, value_dim)
+        for r in range(rows):
+            pos = int(positions[r])
+            page = int(block_table[int(row_req[r]), pos // page_size])
+            k_cache[page, :, pos % page_size] = k[r]
+            v_cache[page, :, pos % page_size] = v[r]
+
+    def sink_window_attention(self, q, num_heads, num_kv_heads, key_dim, value_dim, k_cache, v_cache, block_table,
+                              page_size, positions, row_req, window, keep_first, sink, scale, out):
+        self._count("sink_window_attention")
+        rows = q.shape[0]
+        qf = q.float().view(rows, num_heads, key_dim)
+        group = num_heads // num_kv_heads
+        for r in range(rows):
+            i, b = int(positions[r]), int(row_req[r])
+            lo = max(0, i - window + 1) if window else 0
+            js = list(range(min(int(keep_first or 0), lo))) + list(range(lo, i + 1))
+            pages = torch.tensor([int(block_table[b, j // page_size]) for j in js])
+            offs = torch.tensor([j % page_size for j in js])
+            k = k_cache[pages, :, offs].float()          # [keys, G, D]
+            v = v_cache[pages, :, offs].float()
+            for h in range(num_heads):
+                s = (k[:, h // group] @ qf[r, h]) * scale
+                if sink is not None:
+                    s = torch.cat([s, sink[h].float().view(1)])
+                w = torch.softmax(s, 0)[:len(js)]
+                out[r, h * value_dim:(h + 1) * value_dim] = (w @ v[:, h // group]).to(out.dtype)
+
+    SCAN_SLICE = 16
+
+    def gla_slices(self, key_dim):
+        return (key_dim + self.SCAN_SLICE - 1) // self.SCAN_SLICE
+
+    def gla_decay(self, low, rank, w2, bias, tau, decay):
+        self._count("gla_decay")
+        z = low[:, :rank].float() @ w2.float().t()
+        if bias is not None:
+            z = z + bias.float()
+        decay.copy_(torch.exp(torch.nn.functional.logsigmoid(z) / tau))
+
+    def gla_scan(self, proj, off_q, off_k, off_v, decay, q_scale, num_heads, key_dim, value_dim, state, q_start,
+                 req_rows, n_reqs, parts):
+        self._count("gla_scan")
+        H, D, E, S = num_heads, key_dim, value_dim, self.SCAN_SLICE
+        for b in range(n_reqs):
+            slot = int(req_rows[b])
+            st = state[slot]
+            for t in range(int(q_start[b]), int(q_start[b + 1])):
+                q = proj[t, off_q:off_q + H * D].view(H, D) * q_scale
+                k = proj[t, off_k:off_k + H * D].view(H, D)
+                v = proj[t, off_v:off_v + H * E].view(H, E)
+                st.mul_(decay[t].view(H, D, 1)).add_(k.unsqueeze(-1) * v.unsqueeze(-2))
+                o = st * q.unsqueeze(-1)                        # [H, D, E]
+                for s in range(parts.shape[2]):
+                    parts[t, :, s] = o[:, s * S:(s + 1) * S].sum(1)
+
+    def gla_output(self, parts, num_heads, key_dim, value_dim, weight, eps, proj, off_gate, out):
+        self._count("gla_output")
+        o = parts.sum(2)                                        # [rows, H, E]
+        y = o / torch.sqrt((o * o).mean(-1, keepdim=True) + eps) * weight.float()
+        g = proj[:, off_gate:off_gate + num_heads * value_dim].float().view(-1, num_heads, value_dim)
+        out.copy_((y * g * torch.sigmoid(g)).reshape(out.shape).to(out.dtype))
 
     # ------------------------------------------------- fused few-row kernels
     FUSED_MAX_ROWS = 64
