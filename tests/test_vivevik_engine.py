@@ -1,0 +1,176 @@
+"""Vivevik through the engine (its cache and state manager, step function, scheduler) against
+the plain implementation: once on the CPU with the per-kernel PyTorch references in place
+of the HIP kernels, once on the GPU with the kernels themselves."""
+import pytest
+import torch
+
+import helpers as H
+import vivevik_cases as V
+import plain_vivevik
+from emu_ops import EmuOps
+
+BACKENDS = ["emu", pytest.param("hip", marks=pytest.mark.gpu)]
+LENGTHS = {"P": [1, 9, 37, 83], "Q": [2, 30, 71], "R": [5, 52, 90]}
+# Logits have a standard deviation of about 2.  float32: sums in another order than the float64
+# plain implementation.  bfloat16: the scores of these configurations are sharp on purpose
+# (standard deviation 5 to 8), so rounding queries and keys to 8 bits of mantissa moves a few
+# near-ties by whole weights: the kernels' references in float32 arithmetic with the same roundings
+# are off the plain implementation by 0.054 in the root mean square over all logits and 0.58
+# at most (configuration P); the bounds are twice that.
+TOL = {"f32": 2e-4}
+TOL_BF16 = (0.11, 1.2)      # (root mean square, max)
+
+
+def engine_of(name, backend, dtype, **kw):
+    if backend == "emu":
+        return V.make_engine(name, 1, dtype, ops=EmuOps(), device="cpu", **kw)
+    return V.make_engine(name, 1, dtype, **kw)
+
+
+def sequences_of(name, lengths=None):
+    cfg = V.config_of(name)
+    return {f"r{i}": V.random_ids(cfg, n, 10 + i) for i, n in enumerate(lengths or LENGTHS[name])}
+
+
+def all_decode(seqs):
+    """Every token in a step of its own: what a prompt's step computed must equal this."""
+    steps = []
+    for rid, ids in seqs.items():
+        steps += [([(rid, 1, True)], [rid] if i == len(ids) - 1 else []) for i in range(len(ids))]
+    return steps
+
+
+CUTS = {"whole": H.steps_whole, "decode": H.steps_prefill_then_decode, "token by token": all_decode,
+        "portions": H.steps_portions,
+        "small portions": lambda s: H.steps_portions(s, sizes=(2, 3, 2, 5, 2, 2, 17, 2)),
+        "mixed": H.steps_mixed}
+
+
+@pytest.mark.parametrize("backend", BACKENDS)
+@pytest.mark.parametrize("name", ["P", "Q", "R"])
+@pytest.mark.parametrize("cut", list(CUTS))
+def test_every_cut_matches_plain(backend, name, cut):
+    """Whole prompts, decoding, portions down to two tokens, mixed batches with few pages and
+    slots (freed and used again): the logits at every position are the plain implementation's."""
+    seqs = sequences_of(name)
+    want = {rid: V.plain_logits(name, 1, ids) for rid, ids in seqs.items()}
+    engine = engine_of(name, backend, "f32", page_size=16, num_pages=14, max_requests=3 if cut == "mixed" else 2)
+    steps = CUTS[cut](seqs) if cut != "mixed" else H.steps_mixed(seqs, max_live=3)
+    got = H.run_trace(engine, seqs, steps)
+    bad = H.first_wrong(got, want, TOL["f32"])
+    assert bad is None, f"first wrong logits at (request, position, error) = {bad}"
+    engine.cache.check()
+    m = engine.cache.metrics()
+    assert m["rows_used"] == 0 and all(g["pages_used"] == 0 for g in m["groups"])
+
+
+@pytest.mark.parametrize("backend", BACKENDS)
+@pytest.mark.parametrize("name", ["P", "Q", "R"])
+def test_bfloat16_mixed_batches(backend, name):
+    seqs = sequences_of(name)
+    want = {rid: V.plain_logits(name, 1, ids) for rid, ids in seqs.items()}
+    engine = engine_of(name, backend, "bf16", page_size=16, num_pages=14, max_requests=3)
+    got = H.run_trace(engine, seqs, H.steps_mixed(seqs, max_live=3))
+    diff = torch.cat([got[rid].double() - want[rid] for rid in got])
+    assert not torch.isnan(diff).any()
+    rms, worst = float(diff.pow(2).mean().sqrt()), float(diff.abs().max())
+    assert rms < TOL_BF16[0] and worst < TOL_BF16[1], (rms, worst)
+
+
+@pytest.mark.parametrize("backend", BACKENDS)
+def test_window_pages_are_given_back_and_the_kept_prefix_stays(backend):
+    """A long decode through windows that cross many pages: pages behind the window go back to
+    the pool while the pages of the kept first positions stay, and the logits stay right."""
+    name = "P"
+    cfg = V.config_of(name)
+    ids = V.random_ids(cfg, 150, 5)
+    engine = engine_of(name, backend, "f32", page_size=16, num_pages=16, max_requests=1)
+    req = engine.open("long")
+    want = V.plain_logits(name, 1, ids)
+    out = engine.step([H.lab.StepEntry(req, ids[:20], [19])]).float().cpu()
+    assert float((out[0].double() - want[19]).abs().max()) < TOL["f32"]
+    for i in range(20, len(ids)):
+        out = engine.step([H.lab.StepEntry(req, [ids[i]], [0])]).float().cpu()
+        assert float((out[0].double() - want[i]).abs().max()) < TOL["f32"], f"decoded position {i}"
+    held = {gi: [lp for lp, p in enumerate(pages) if p >= 0] for gi, pages in enumerate(req.pages)}
+    groups = engine.cache.groups
+    for gi, g in enumerate(groups):
+        if g.window is not None and g.window < 100:
+            assert held[gi][0] == 0, "the page of the kept first positions was given back"
+            assert len(held[gi]) < len(req.pages[gi]), "no page behind the window was given back"
+    engine.close(req)
+    engine.cache.check()
+
+
+@pytest.mark.parametrize("backend", BACKENDS)
+def test_a_slot_used_again_starts_from_zero(backend):
+    """The recurrent state of a finished request must not leak into the one that gets its slot."""
+    name = "Q"
+    cfg = V.config_of(name)
+    engine = engine_of(name, backend, "f32", max_requests=1)
+    first, second = V.random_ids(cfg, 40, 1), V.random_ids(cfg, 25, 2)
+    a = engine.open("a")
+    engine.step([H.lab.StepEntry(a, first, [])])
+    engine.close(a)
+    b = engine.open("b")
+    assert b.row == a.row
+    out = engine.step([H.lab.StepEntry(b, second, list(range(len(second))))]).float().cpu()
+    err = float((out.double() - V.plain_logits(name, 1, second)).abs().max())
+    assert err < TOL["f32"], err
+    engine.close(b)
+
+
+@pytest.mark.parametrize("backend", BACKENDS)
+@pytest.mark.parametrize("name", ["P", "Q"])
+def test_greedy_generation_through_the_scheduler(backend, name):
+    cfg = V.config_of(name)
+    tensors = V.make_tensors(cfg, 1)
+    prompts = [V.random_ids(cfg, n, 40 + n) for n in (3, 17, 30)]
+    engine = engine_of(name, backend, "f32", page_size=16, num_pages=24, max_requests=2, max_batch_tokens=16)
+    got = engine.generate(prompts, max_new_tokens=12)
+    for prompt, tokens in zip(prompts, got):
+        ids = list(prompt)
+        for n, token in enumerate(tokens):
+            logits = plain_vivevik.forward(ids, tensors, cfg.to_dict())[-1]
+            best = int(logits.argmax())
+            assert token == best or float(logits[best] - logits[token]) < 2 * TOL["f32"], \
+                f"generated token {n} is {token}, the plain implementation's is {best}"
+            ids.append(token)
+    m = engine.cache.metrics()
+    assert m["rows_used"] == 0 and all(g["pages_used"] == 0 for g in m["groups"])
+
+
+def test_configuration_round_trip_and_errors():
+    for name, raw in V.CONFIGS.items():
+        cfg = V.config_of(name)
+        again = H.lab.VivevikConfig.from_dict(cfg.to_dict())
+        assert again == cfg
+        arch = H.lab.config.architecture_of(raw)
+        assert arch.name == "Vivevik"
+    bad = dict(V.CONFIGS["R"], layers=[dict(V.CONFIGS["R"]["layers"][1])])
+    with pytest.raises(H.lab.ConfigError):
+        H.lab.VivevikConfig.from_dict(bad)          # kv_from names no earlier layer
+    with pytest.raises(H.lab.ConfigError):
+        H.lab.VivevikConfig.from_dict(dict(V.CONFIGS["Q"], layers=[dict(type="conv", mixer=dict(heads=1, dim=1, vdim=1))]))
+
+
+def test_the_rank_of_the_decays_is_read_from_the_tensors(tmp_path):
+    """A configuration that names no rank takes whatever the model file's tensors have."""
+    raw = dict(V.CONFIGS["Q"])
+    cfg = V.config_of("Q")
+    tensors = V.make_tensors(cfg, 3)
+    no_rank = {**raw, "layers": [{**l, "mixer": {k: v for k, v in l["mixer"].items() if k != "rank"}}
+                                 for l in raw["layers"]]}
+    cfg2 = H.lab.VivevikConfig.from_dict(no_rank)
+    engine = H.lab.Engine(config=cfg2, tensors=tensors.items(), dtype="f32", ops=EmuOps(), device="cpu",
+                          page_size=16, num_pages=8, max_requests=1, max_batch_tokens=64, max_seq_len=64)
+    ids = V.random_ids(cfg, 20, 0)
+    req = engine.open("x")
+    out = engine.step([H.lab.StepEntry(req, ids, [19])]).float()
+    want = plain_vivevik.forward(ids, tensors, cfg.to_dict())[-1]
+    assert float((out[0].double() - want).abs().max()) < TOL["f32"]
+    # the two factors must fit each other
+    tensors["l0.mix.a2"] = tensors["l0.mix.a2"][:, :3].contiguous()
+    with pytest.raises(ValueError):
+        H.lab.Engine(config=cfg2, tensors=tensors.items(), dtype="f32", ops=EmuOps(), device="cpu",
+                     page_size=16, num_pages=8, max_requests=1, max_batch_tokens=64, max_seq_len=64)
