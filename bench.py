@@ -3,6 +3,7 @@
     python bench.py [--gpus 1] [--steps K] [--warmup W] [--batch B] [--context S]
                     [--shape 0.5b|7b|32b] [--layers L] [--dtype bf16|f32]
     python bench.py --mixed [--shape 7b] [--requests 64] [--chunk 512] [--outputs 64]
+    python bench.py --design vivevik [--size small|medium|large] [--context 2048]
 
 Default: the layer sizes of the Qwen2.5-0.5B shape with seeded random weights,
 batch 8, context 4096, bfloat16.  A "step" is one decode step of the whole
@@ -36,6 +37,11 @@ back).  One JSON line is printed: decoded tokens a second as ``value``, plus
 ``--profile``: for runs under ``rocprofv3``: collection is paused (rocTX) except around the
 timed steps, so that the profile holds those and not the filling of the caches
 (rust/engine/benches/qwen2.rs:110-114, 175-179, 297-301).
+
+``--design vivevik``: prefill and decode throughput of the Vivevik design (gated linear
+attention layers beside windowed attention layers with a sink, some of which read an earlier
+layer's keys and values) at layer sizes of real models, beside the Qwen2 decoder with the same
+width, heads, feed-forward width and number of layers; one JSON line, a record per size.
 
 ``--mixed``: many requests with prompts of different lengths go through the
 scheduler with a small token budget, so that portions of prompts run beside the
@@ -92,6 +98,105 @@ def prefill_flops(cfg, tokens):
     per_token_layer = 2 * (h * (q + 2 * kv) + q * h + 3 * h * i)
     attention_layer = 4 * (tokens * (tokens + 1) // 2) * q
     return cfg.num_hidden_layers * (tokens * per_token_layer + attention_layer) + 2 * h * v
+
+
+# Layer sizes for ``--design vivevik``: (width, heads, kv heads, head size, feed-forward width,
+# layers).  Layers come in threes: a recurrent layer without a feed-forward, an attention layer
+# with keys and values of its own, and one that reads the former's; windows of 1,024 positions
+# that keep the first four.
+DESIGN_SIZES = {"small": (896, 14, 2, 64, 4864, 12), "medium": (2048, 16, 2, 128, 11008, 12),
+                "large": (3584, 28, 4, 128, 18944, 6)}
+DESIGN_VOCAB = 32000
+DESIGN_WINDOW, DESIGN_KEEP = 1024, 4
+
+
+def vivevik_config(size):
+    import llm_inference_lab_amd as lab
+    width, heads, kv, dim, ff, layers = DESIGN_SIZES[size]
+    listed = []
+    for i in range(layers):
+        if i % 3 == 0:
+            listed.append(dict(type="gla", mlp=None,
+                               mixer=dict(heads=width // 128, dim=64, vdim=128, tau=16.0, rank=16)))
+        else:
+            mixer = dict(heads=heads, kv_heads=kv, dim=dim, vdim=dim, scale=dim ** -0.5,
+                         mask=dict(size=DESIGN_WINDOW, keep_first=DESIGN_KEEP))
+            if i % 3 == 2:
+                mixer["kv_from"] = i - 1
+            listed.append(dict(type="attention", mixer=mixer, mlp=dict(kind="dense", ff=ff)))
+    return lab.VivevikConfig.from_dict(dict(architecture="Vivevik", vocab=DESIGN_VOCAB, width=width,
+                                            norm=dict(eps=1e-6), layers=listed))
+
+
+def vivevik_flops(cfg, tokens):
+    """Multiply-adds times two of one prompt of ``tokens`` positions (products and attention;
+    the recurrence counts its state update and its read-out)."""
+    w, total = cfg.width, 0
+    for l in cfg.layers:
+        if l.type == "gla":
+            qk, v = l.heads * l.dim, l.heads * l.vdim
+            total += tokens * 2 * (w * (2 * qk + 2 * v + (l.rank or 16)) + v * w + (l.rank or 16) * qk)
+            total += tokens * 4 * l.heads * l.dim * l.vdim
+        else:
+            q, k, v = l.heads * l.dim, l.kv_heads * l.dim, l.kv_heads * l.vdim
+            total += tokens * 2 * (w * (q + (k + v if l.kv_from is None else 0)) + l.heads * l.vdim * w)
+            seen = sum(min(i + 1, (l.window or tokens) + l.keep_first) for i in range(tokens))
+            total += 2 * seen * l.heads * (l.dim + l.vdim)
+        if l.mlp is not None:
+            total += tokens * 4 * w * l.mlp.ff
+    return total + 2 * w * cfg.vocab
+
+
+def design_run(args):
+    """``--design vivevik``: both models at each size, one after the other on the same GPU."""
+    import types
+    import torch
+    import llm_inference_lab_amd as lab
+    from llm_inference_lab_amd.config import get_architecture
+    from llm_inference_lab_amd.engine.model import CausalLM
+    context = args.context or 2048
+    batches = sorted({8, 64})
+    record = {}
+    for size in ([args.size] if args.size else list(DESIGN_SIZES)):
+        width, heads, kv, dim, ff, layers = DESIGN_SIZES[size]
+        qwen = lab.Qwen2Config.from_dict(dict(COMMON, vocab_size=DESIGN_VOCAB, hidden_size=width, intermediate_size=ff,
+                                              num_hidden_layers=layers, num_attention_heads=heads,
+                                              num_key_value_heads=kv, head_dim=dim, tie_word_embeddings=True))
+        record[size] = {"width": width, "heads": heads, "kv_heads": kv, "head_dim": dim, "ff": ff, "layers": layers,
+                        "context": context, "window": DESIGN_WINDOW}
+        for label, cfg in (("vivevik", vivevik_config(size)), ("qwen2", qwen)):
+            expected = CausalLM(get_architecture(cfg.architecture).build_spec(cfg)).tensor_specs()
+            arch = get_architecture(cfg.architecture)
+            drawn = (arch.random_init(cfg, expected, 0, torch.bfloat16) if arch.random_init is not None
+                     else random_weights_on_the_gpu(expected, 0))
+            engine = lab.Engine(config=cfg, tensors=drawn, dtype=args.dtype, device="cuda:0", page_size=PAGE,
+                                max_cache_tokens=max(batches) * (context + PAGE), max_requests=max(batches),
+                                max_batch_tokens=FILL_TOKENS, max_seq_len=context + PAGE,
+                                graph=False if args.no_graph else args.graph)
+            view = types.SimpleNamespace(vocab_size=engine.spec.vocab_size)
+            runs = Runs(engine, view, context, args.dtype, args.samples)
+            flops = vivevik_flops(cfg, args.prefill_tokens) if label == "vivevik" else prefill_flops(cfg, args.prefill_tokens)
+            out = {"prefill": runs.prefill(args.prefill_tokens, flops=flops),
+                   "weight_bytes_per_step": engine.weight_bytes_per_step()}
+            # what a decode step has to move: the weights once, of every request the cache its
+            # layers still see (a windowed group: the window and the kept prefix) and its
+            # recurrent states, read and written
+            state = 2 * sum(t[0].numel() * t.element_size() for per in engine.cache.state.values() for t in per.values())
+            for b in batches:
+                seconds, live, ms = runs.decode_samples(b, args.steps, args.warmup)
+                seen = sum(len(g.entries) * g.spec.bytes_per_token(engine.cache.dtype)
+                           * min(live / b, (g.window + g.spec.keep_first) if g.window else live / b)
+                           for g in engine.cache.groups)
+                moved = out["weight_bytes_per_step"] + b * (seen + state)
+                out[f"decode_b{b}"] = {"value": round(b * args.steps / seconds, 1), "ms_per_step": ms["median"],
+                                       "hbm_frac": round(moved / (seconds / args.steps) / (HBM_PEAK_GBS * 1e9), 4)}
+            record[size][label] = out
+            del engine, runs
+            torch.cuda.empty_cache()
+        print(f"[bench] {size}: {json.dumps(record[size])}", file=sys.stderr, flush=True)
+    print(json.dumps({"metric": "design_throughput", "design": "vivevik", "beside": "qwen2", "dtype": args.dtype,
+                      "data": "synthetic", "unit": "tokens/s", "prefill_tokens": args.prefill_tokens,
+                      "sizes": record}))
 
 
 def random_weights_on_the_gpu(expected, seed):
@@ -334,7 +439,7 @@ class Runs:
         times.sort()
         return round(times[len(times) // 2], 4), round(times[min(len(times) - 1, int(len(times) * 0.95))], 4)
 
-    def prefill(self, tokens=2048, repeats=None):
+    def prefill(self, tokens=2048, repeats=None, flops=None):
         """One prompt in one step, logits at its last place: one untimed run, then the median
         of ``repeats`` (at least ``--samples``, at least three) with a fresh request each."""
         from llm_inference_lab_amd.engine.step import StepEntry
@@ -356,7 +461,7 @@ class Runs:
             self.engine.close(req)
         ms = spread([t * 1e3 for t in times], 3)
         median = ms["median"] * 1e-3
-        flops = prefill_flops(self.cfg, tokens)
+        flops = flops if flops is not None else prefill_flops(self.cfg, tokens)
         out = {"value": round(tokens / median, 1), "tokens": tokens, "ms": ms["median"],
                "frac": round(flops / median / PEAK_FLOPS[self.dtype], 4), "ms_min": ms["min"], "ms_max": ms["max"],
                "samples": ms["n"]}
@@ -600,6 +705,9 @@ def main():
                     help="fix a choice of the kernels for the whole run, to compare variants: a keyword of "
                          "engine.ops.debug.force, values separated by ':' (attention_splits=64:8, "
                          "attention_merge_kernel=64, gemm_tile=129)")
+    ap.add_argument("--design", choices=["vivevik"], default=None,
+                    help="throughput of another design beside the Qwen2 decoder of equal size")
+    ap.add_argument("--size", choices=sorted(DESIGN_SIZES), default=None, help="--design: one size only")
     ap.add_argument("--side", choices=["7b", "32b", "f32", "peaks"], help=argparse.SUPPRESS)
     args = ap.parse_args()
     if args.gpus != 1:
@@ -610,6 +718,9 @@ def main():
         args.graph = True
     if args.side:
         side_run(args)
+        return
+    if args.design:
+        design_run(args)
         return
 
     # The other shapes and the other dtype are points of the default line: each runs as a
