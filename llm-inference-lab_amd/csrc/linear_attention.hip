@@ -43,75 +43,168 @@ extern "C" int llmlab_gla_decay(const float* low, int ld, int rows, int rank, co
 }
 
 // ------------------------------------------------------------------------ scan
-// Block (request b, head h, slab of value columns).  Thread (s, e) keeps the SLICE rows
-// s * SLICE .. of column e of the head's state in registers, walks the request's rows of
-// this step in order, and leaves its part of o_t in parts[row, h, s, e]; the output kernel
-// adds the parts of the slices.  Threads never talk to each other, so a token costs no
-// barrier; the loads of a token do not depend on the state, so they run ahead of the sums.
-// The state is read from the request's slot before the first row and written back after
-// the last.
-__global__ __launch_bounds__(1024) void gla_scan_kernel(
-    const float* __restrict__ proj, int ld, int off_q, int off_k, int off_v, const float* __restrict__ decay,
-    float q_scale, int n_heads, int D, int E, int cols, int slices, float* __restrict__ state,
-    const int* __restrict__ q_start, const int* __restrict__ req_rows, float* __restrict__ parts) {
-  const int b = blockIdx.x, h = blockIdx.y;
-  const int e = blockIdx.z * cols + (int)(threadIdx.x % cols);
-  const int s = threadIdx.x / cols;
-  if (e >= E || s >= slices) return;
-  const int d0 = s * SLICE;
-  float S[SLICE];
-  float* st = state + (((size_t)req_rows[b] * n_heads + h) * D + d0) * E + e;
+// Thread (s, e) of a block keeps the SLICE rows s * SLICE .. of column e of one head's state in
+// registers, walks a run of rows in order, and leaves its part of o_t in parts[row, h, s, e];
+// the output kernel adds the parts of the slices.  Threads never talk to each other, so a
+// token costs no barrier; the loads of a token do not depend on the state, so they run
+// ahead of the sums.
+//
+// WHOLE: a block takes all the rows that request blockIdx.x brings to the step: the state
+// comes from the request's slot and goes back there.  That is the kernel of decode steps
+// and of short portions.
+//
+// Long portions are cut into chunks of `chunk` rows that run side by side, in three passes
+// (the recurrence is linear in the state: S_end = P * S_start + L with P the product of the
+// chunk's decays and L the state the chunk builds from zero):
+//   LOCAL  per chunk: L and P, from a zero state, no outputs;
+//   carry  per request, chunk after chunk: S_start[c], and the request's slot at the end;
+//   FINISH per chunk: the rows again from S_start[c], now with outputs.
+// All of it in float32; the result differs from the row-by-row recurrence by rounding only.
+enum { SCAN_WHOLE = 0, SCAN_LOCAL = 1, SCAN_FINISH = 2 };
+
+struct ScanArgs {
+  const float* proj; int ld, off_q, off_k, off_v;
+  const float* decay; float q_scale; int n_heads, D, E, cols, slices;
+  float* state; const int* q_start; const int* req_rows; float* parts;
+  int n_reqs, chunk; float* chunk_state; float* chunk_decay;      // [chunks, heads, D, E] and [chunks, heads, D]
+};
+
+// Which request and which rows the chunk `index` of the step covers (chunks are counted
+// request after request); false if the step has fewer chunks.
+__device__ __forceinline__ bool find_chunk(const ScanArgs& a, int index, int& first, int& last) {
+  int before = 0;
+  for (int b = 0; b < a.n_reqs; ++b) {
+    const int lo = a.q_start[b], hi = a.q_start[b + 1];
+    const int n = (hi - lo + a.chunk - 1) / a.chunk;
+    if (index < before + n) {
+      first = lo + (index - before) * a.chunk;
+      last = first + a.chunk < hi ? first + a.chunk : hi;
+      return true;
+    }
+    before += n;
+  }
+  return false;
+}
+
+template <int MODE, bool UNIFORM>
+__global__ __launch_bounds__(1024) void gla_scan_kernel(ScanArgs a) {
+  const int h = blockIdx.y;
+  const int e = blockIdx.z * a.cols + (int)(threadIdx.x % a.cols);
+  // UNIFORM: a wave lies within one slice (cols a multiple of 64), so the slice's decays,
+  // keys and queries are the same for all its lanes and can come through the scalar unit
+  const int s = UNIFORM ? __builtin_amdgcn_readfirstlane((int)(threadIdx.x / a.cols)) : (int)(threadIdx.x / a.cols);
+  int first, last;
+  if (MODE == SCAN_WHOLE) {
+    first = a.q_start[blockIdx.x];
+    last = a.q_start[blockIdx.x + 1];
+  } else if (!find_chunk(a, blockIdx.x, first, last)) {
+    return;
+  }
+  if (e >= a.E || s >= a.slices) return;
+  const int D = a.D, E = a.E, d0 = s * SLICE;
+  float S[SLICE], P[SLICE];
+  float* st = MODE == SCAN_WHOLE ? a.state + (((size_t)a.req_rows[blockIdx.x] * a.n_heads + h) * D + d0) * E + e
+                                 : a.chunk_state + (((size_t)blockIdx.x * a.n_heads + h) * D + d0) * E + e;
 #pragma unroll
-  for (int i = 0; i < SLICE; ++i) S[i] = d0 + i < D ? st[(size_t)i * E] : 0.f;
-  const int first = q_start[b], last = q_start[b + 1];
+  for (int i = 0; i < SLICE; ++i) {
+    S[i] = (MODE != SCAN_LOCAL && d0 + i < D) ? st[(size_t)i * E] : 0.f;
+    P[i] = 1.f;
+  }
   const bool whole = d0 + SLICE <= D;
   for (int t = first; t < last; ++t) {
-    const float* row = proj + (size_t)t * ld;
-    const float* qp = row + off_q + h * D + d0;
-    const float* kp = row + off_k + h * D + d0;
-    const float* ap = decay + ((size_t)t * n_heads + h) * D + d0;
-    const float v = row[off_v + h * E + e];
+    const float* row = a.proj + (size_t)t * a.ld;
+    const float* qp = row + a.off_q + h * D + d0;
+    const float* kp = row + a.off_k + h * D + d0;
+    const float* ap = a.decay + ((size_t)t * a.n_heads + h) * D + d0;
+    const float v = row[a.off_v + h * E + e];
     float acc = 0.f;
-    if (whole) {
 #pragma unroll
-      for (int i = 0; i < SLICE; ++i) {
+    for (int i = 0; i < SLICE; ++i) {
+      if (whole || d0 + i < D) {
         S[i] = fmaf(ap[i], S[i], kp[i] * v);
-        acc = fmaf(S[i], qp[i] * q_scale, acc);
-      }
-    } else {
-#pragma unroll
-      for (int i = 0; i < SLICE; ++i) {
-        if (d0 + i < D) {
-          S[i] = fmaf(ap[i], S[i], kp[i] * v);
-          acc = fmaf(S[i], qp[i] * q_scale, acc);
-        }
+        if (MODE == SCAN_LOCAL) P[i] *= ap[i];
+        else acc = fmaf(S[i], qp[i] * a.q_scale, acc);
       }
     }
-    parts[(((size_t)t * n_heads + h) * slices + s) * E + e] = acc;
+    if (MODE != SCAN_LOCAL) a.parts[(((size_t)t * a.n_heads + h) * a.slices + s) * E + e] = acc;
   }
+  if (MODE == SCAN_FINISH) return;
 #pragma unroll
   for (int i = 0; i < SLICE; ++i)
     if (d0 + i < D) st[(size_t)i * E] = S[i];
+  if (MODE == SCAN_LOCAL && e == 0) {
+    float* pd = a.chunk_decay + ((size_t)blockIdx.x * a.n_heads + h) * D + d0;
+#pragma unroll
+    for (int i = 0; i < SLICE; ++i)
+      if (d0 + i < D) pd[i] = P[i];
+  }
+}
+
+// One thread per element (h, d, e) of a request's state, chunk after chunk:
+// chunk_state[c] <- the state before chunk c; the slot <- the state after the last chunk.
+__global__ __launch_bounds__(256) void gla_carry_kernel(ScanArgs a) {
+  const int b = blockIdx.y;
+  const size_t per = (size_t)a.n_heads * a.D * a.E;
+  const size_t i = (size_t)blockIdx.x * blockDim.x + threadIdx.x;
+  if (i >= per) return;
+  int before = 0;
+  for (int r = 0; r < b; ++r) before += (a.q_start[r + 1] - a.q_start[r] + a.chunk - 1) / a.chunk;
+  const int n = (a.q_start[b + 1] - a.q_start[b] + a.chunk - 1) / a.chunk;
+  float* slot = a.state + (size_t)a.req_rows[b] * per + i;
+  float S = *slot;
+  const size_t hd = i / a.E;
+  for (int c = before; c < before + n; ++c) {
+    float* l = a.chunk_state + (size_t)c * per + i;
+    const float built = *l;
+    *l = S;
+    S = fmaf(a.chunk_decay[(size_t)c * a.n_heads * a.D + hd], S, built);
+  }
+  *slot = S;
 }
 
 extern "C" int llmlab_gla_slices(int D) { return (D + SLICE - 1) / SLICE; }
 
 // proj [rows, ld] float32 holds q at off_q (heads * D), k at off_k, v at off_v (heads * E);
 // decay [rows, heads * D]; state [slots, heads, D, E]; parts [rows, heads, slices, E].
+// chunk > 0: the three-pass form over chunks of so many rows; chunk_state then holds
+// max_chunks * heads * D * E floats and chunk_decay max_chunks * heads * D, with max_chunks >=
+// rows / chunk + n_reqs.
 extern "C" int llmlab_gla_scan(const float* proj, int ld, int off_q, int off_k, int off_v, const float* decay,
                                float q_scale, int n_heads, int D, int E, float* state, const int* q_start,
-                               const int* req_rows, int n_reqs, float* parts, hipStream_t stream) {
+                               const int* req_rows, int n_reqs, float* parts, int rows, int chunk,
+                               float* chunk_state, float* chunk_decay, int max_chunks, hipStream_t stream) {
   LLMLAB_REQUIRE(n_reqs >= 0 && n_heads > 0 && D > 0 && E > 0, "gla_scan: bad sizes reqs=%d heads=%d D=%d E=%d", n_reqs,
                  n_heads, D, E);
   const int slices = (D + SLICE - 1) / SLICE;
   int cols = E < 64 ? E : 64;
   while (cols > 1 && slices * cols > 1024) cols /= 2;
   LLMLAB_REQUIRE(slices * cols <= 1024, "gla_scan: %d key channels per head are more than a block holds", D);
-  LLMLAB_REQUIRE(n_heads <= 65535 && (E + cols - 1) / cols <= 65535, "gla_scan: too many heads or columns");
+  LLMLAB_REQUIRE(n_heads <= 65535 && (E + cols - 1) / cols <= 65535 && n_reqs <= 65535,
+                 "gla_scan: too many heads, columns or requests");
   if (n_reqs == 0) return 0;
-  dim3 grid(n_reqs, n_heads, (E + cols - 1) / cols), block(slices * cols);
-  hipLaunchKernelGGL(gla_scan_kernel, grid, block, 0, stream, proj, ld, off_q, off_k, off_v, decay, q_scale, n_heads, D,
-                     E, cols, slices, state, q_start, req_rows, parts);
+  ScanArgs a{proj, ld, off_q, off_k, off_v, decay, q_scale, n_heads, D, E, cols, slices, state, q_start, req_rows, parts,
+             n_reqs, chunk, chunk_state, chunk_decay};
+  const bool uniform = cols == 64;
+  dim3 block(slices * cols);
+  const unsigned slabs = (E + cols - 1) / cols;
+#define LLMLAB_SCAN(MODE, GRIDX)                                                                              \
+  do {                                                                                                        \
+    if (uniform) hipLaunchKernelGGL((gla_scan_kernel<MODE, true>), dim3(GRIDX, n_heads, slabs), block, 0, stream, a); \
+    else hipLaunchKernelGGL((gla_scan_kernel<MODE, false>), dim3(GRIDX, n_heads, slabs), block, 0, stream, a);  \
+  } while (0)
+  if (chunk <= 0) {
+    LLMLAB_SCAN(SCAN_WHOLE, n_reqs);
+  } else {
+    const int chunks = rows / chunk + n_reqs;
+    LLMLAB_REQUIRE(chunk_state && chunk_decay && max_chunks >= chunks,
+                   "gla_scan: %d rows of %d requests in chunks of %d need room for %d chunks, got %d", rows, n_reqs,
+                   chunk, chunks, max_chunks);
+    LLMLAB_SCAN(SCAN_LOCAL, chunks);
+    const size_t per = (size_t)n_heads * D * E;
+    hipLaunchKernelGGL(gla_carry_kernel, dim3((unsigned)((per + 255) / 256), n_reqs), dim3(256), 0, stream, a);
+    LLMLAB_SCAN(SCAN_FINISH, chunks);
+  }
+#undef LLMLAB_SCAN
   LLMLAB_LAUNCH_CHECK("gla_scan");
   return 0;
 }

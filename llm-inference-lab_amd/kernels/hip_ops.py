@@ -1000,7 +1000,8 @@ class HipOps:
                 lib.llmlab_gla_slices.argtypes = [_c_int]
                 lib.llmlab_gla_slices.restype = _c_int
                 lib.llmlab_gla_scan.argtypes = [_c_ptr, _c_int, _c_int, _c_int, _c_int, _c_ptr, _c_float, _c_int, _c_int,
-                                                _c_int, _c_ptr, _c_ptr, _c_ptr, _c_int, _c_ptr, _c_ptr]
+                                                _c_int, _c_ptr, _c_ptr, _c_ptr, _c_int, _c_ptr, _c_int, _c_int, _c_ptr,
+                                                _c_ptr, _c_int, _c_ptr]
                 lib.llmlab_gla_scan.restype = _c_int
                 lib.llmlab_gla_output.argtypes = [_c_ptr, _c_int, _c_int, _c_int, _c_int, _c_ptr, _c_float, _c_ptr,
                                                   _c_int, _c_int, _c_ptr, _c_int, _c_ptr]
@@ -1123,12 +1124,29 @@ class HipOps:
         self._call(lib.llmlab_gla_decay, self._ptr(low), low.stride(0), rows, int(rank), self._ptr(w2),
                    self._ptr(bias), float(tau), self._ptr(decay), channels, self._stream(), lib=lib)
 
+    def gla_scan_chunk(self, rows: int, longest: int, num_heads: int, value_dim: int) -> int:
+        """Into chunks of how many rows the scan cuts a step whose longest request brings
+        ``longest`` rows (0: every request's rows in one run).  Chunks run side by side at the
+        price of walking the rows twice, so short runs stay whole, and the chunks are as long
+        as still gives every compute unit a few blocks."""
+        if longest < 2 * self.rules.scan_min_chunk:
+            return 0
+        per_chunk = num_heads * ((value_dim + 63) // 64)
+        chunk = self.rules.scan_max_chunk
+        while chunk > self.rules.scan_min_chunk and (rows // chunk) * per_chunk < 4 * self.num_cus:
+            chunk //= 2
+        return chunk
+
     def gla_scan(self, proj, off_q, off_k, off_v, decay, q_scale, num_heads, key_dim, value_dim, state, q_start,
-                 req_rows, n_reqs, parts) -> None:
+                 req_rows, n_reqs, parts, chunk=0, chunk_state=None, chunk_decay=None) -> None:
         """The recurrence ``S = decay_t * S + k_t v_t^T; o_t = S^T (q_scale q_t)`` over the rows
         ``q_start[b] .. q_start[b + 1]`` of each of the step's ``n_reqs`` requests, on the float32
         state ``state[req_rows[b]]`` ``[heads, key_dim, value_dim]``, which is left updated;
-        ``parts [rows, heads, gla_slices(key_dim), value_dim]`` receives each output in pieces."""
+        ``parts [rows, heads, gla_slices(key_dim), value_dim]`` receives each output in pieces.
+        ``chunk > 0``: every request's rows in chunks of so many that run side by side, their
+        states joined afterwards (``chunk_state [chunks, heads, key_dim, value_dim]`` and
+        ``chunk_decay [chunks, heads, key_dim]`` float32 scratch, ``chunks >= rows // chunk +
+        n_reqs``)."""
         lib = self._mixer_lib("linear_attention")
         for t, name in ((proj, "projections"), (decay, "decays"), (state, "recurrent state"), (parts, "output pieces")):
             self._need(t, name, torch.float32)
@@ -1143,9 +1161,21 @@ class HipOps:
                 or min(off_q, off_k, off_v) < 0
                 or max(off_q + num_heads * key_dim, off_k + num_heads * key_dim, off_v + num_heads * value_dim) > proj.shape[1]):
             raise ValueError("gla_scan: the operands do not fit each other")
+        max_chunks = 0
+        if chunk:
+            self._need(chunk_state, "chunk states", torch.float32)
+            self._need(chunk_decay, "chunk decays", torch.float32)
+            max_chunks = chunk_state.shape[0]
+            if (tuple(chunk_state.shape[1:]) != (num_heads, key_dim, value_dim)
+                    or tuple(chunk_decay.shape) != (max_chunks, num_heads, key_dim)
+                    or max_chunks < rows // chunk + n_reqs):
+                raise ValueError(f"gla_scan: the scratch of the chunks does not fit {rows} rows of {n_reqs} requests "
+                                 f"in chunks of {chunk}")
         self._call(lib.llmlab_gla_scan, self._ptr(proj), proj.stride(0), int(off_q), int(off_k), int(off_v),
                    self._ptr(decay), float(q_scale), num_heads, key_dim, value_dim, self._ptr(state),
-                   self._ptr(q_start), self._ptr(req_rows), int(n_reqs), self._ptr(parts), self._stream(), lib=lib)
+                   self._ptr(q_start), self._ptr(req_rows), int(n_reqs), self._ptr(parts), rows, int(chunk),
+                   self._ptr(chunk_state) if chunk else None, self._ptr(chunk_decay) if chunk else None, max_chunks,
+                   self._stream(), lib=lib)
 
     def gla_output(self, parts, num_heads, key_dim, value_dim, weight, eps, proj, off_gate, out) -> None:
         """``out[r, h] = rmsnorm(sum of parts[r, h]) * weight * silu(gate[r, h])`` with the gate at

@@ -94,6 +94,10 @@ class GatedLinearAttention(Mixer):
         self.b_decay = tensors[t["decay_bias"]].float().contiguous()
         self.norm_weight = tensors[t["out_norm"]].float().contiguous()
 
+    def _min_chunk(self) -> int:
+        rules = getattr(self.ops, "rules", None)
+        return int(getattr(rules, "scan_min_chunk", 16))
+
     def state_spec(self):
         return {"s": ((self.num_heads, self.key_dim, self.value_dim), torch.float32)}
 
@@ -106,12 +110,20 @@ class GatedLinearAttention(Mixer):
         parts = ctx.scratch("linear_attention.parts",
                             (rows, self.num_heads, ops.gla_slices(self.key_dim), self.value_dim), torch.float32)
         state = entry.state["s"]
+        # room for the chunks of a long portion: at most rows / (smallest chunk) + requests
+        most = rows // max(1, self._min_chunk()) + ctx.max_reqs
+        chunk_state = ctx.scratch("linear_attention.chunk_state",
+                                  (most, self.num_heads, self.key_dim, self.value_dim), torch.float32)
+        chunk_decay = ctx.scratch("linear_attention.chunk_decay", (most, self.num_heads, self.key_dim), torch.float32)
 
         def scan():
-            # (how many requests the step has is read when the launch is made, also when it is
-            # made again from a kept sequence of calls)
+            # (how many requests the step has and how long the longest portion is are read when
+            # the launch is made, also when it is made again from a kept sequence of calls)
+            pick = getattr(ops, "gla_scan_chunk", None)
+            chunk = pick(rows, ctx.max_q_len, self.num_heads, self.value_dim) if pick is not None else 0
             ops.gla_scan(proj, o["q_weight"], o["k_weight"], o["v_weight"], decay, self.q_scale, self.num_heads,
-                         self.key_dim, self.value_dim, state, ctx.all_q_start, ctx.all_req_rows, ctx.n_reqs, parts)
+                         self.key_dim, self.value_dim, state, ctx.all_q_start, ctx.all_req_rows, ctx.n_reqs, parts,
+                         chunk, chunk_state if chunk else None, chunk_decay if chunk else None)
         live = getattr(ops, "live", None)
         if live is not None:
             live(scan)

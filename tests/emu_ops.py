@@ -66,7 +66,7 @@ class EmuOps:
         self.calls = {}
         self.fuse = fuse
         import types
-        self.rules = types.SimpleNamespace(min_steps_per_split=8)
+        self.rules = types.SimpleNamespace(min_steps_per_split=8, scan_min_chunk=16, scan_max_chunk=64)
         self._record = None
         self._depth = 0
         for name in self.RECORDED:
@@ -308,9 +308,15 @@ class EmuOps:
             z = z + bias.float()
         decay.copy_(torch.exp(torch.nn.functional.logsigmoid(z) / tau))
 
+    def gla_scan_chunk(self, rows, longest, num_heads, value_dim):
+        return 16 if longest >= 32 else 0
+
     def gla_scan(self, proj, off_q, off_k, off_v, decay, q_scale, num_heads, key_dim, value_dim, state, q_start,
-                 req_rows, n_reqs, parts):
+                 req_rows, n_reqs, parts, chunk=0, chunk_state=None, chunk_decay=None):
+        """(``chunk``: how the kernel spreads the work; the recurrence is the same.)"""
         self._count("gla_scan")
+        if chunk:
+            assert chunk_state.shape[0] >= proj.shape[0] // chunk + n_reqs and chunk_decay.shape[0] == chunk_state.shape[0]
         H, D, E, S = num_heads, key_dim, value_dim, self.SCAN_SLICE
         for b in range(n_reqs):
             slot = int(req_rows[b])

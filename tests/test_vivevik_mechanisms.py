@@ -229,11 +229,14 @@ def test_decays(backend):
 
 @pytest.mark.parametrize("backend", BACKENDS)
 @pytest.mark.parametrize("dtype", DTYPES)
-@pytest.mark.parametrize("heads,D,E", [(2, 24, 16), (1, 16, 1), (3, 40, 72), (2, 7, 130)])
-def test_recurrence_over_portions_and_requests(backend, dtype, heads, D, E):
+@pytest.mark.parametrize("heads,D,E", [(2, 24, 16), (1, 16, 1), (3, 40, 72), (2, 7, 130), (2, 32, 64)])
+@pytest.mark.parametrize("chunk", [0, 16, 5])
+def test_recurrence_over_portions_and_requests(backend, dtype, heads, D, E, chunk):
     """Three requests in one call (a long portion, a single token, two tokens), then the same
     requests again with their states carried, against the plain recurrence over each whole
-    sequence; then the output norm and gate."""
+    sequence; then the output norm and gate.  ``chunk``: the rows of a request cut into chunks
+    that run side by side and are joined afterwards (a last chunk that is not full, requests
+    shorter than a chunk)."""
     ops = ops_of(backend)
     dev = ops.device
     lengths = [(37, 6), (1, 1), (2, 20)]                # (first call, second call) per request
@@ -259,9 +262,12 @@ def test_recurrence_over_portions_and_requests(backend, dtype, heads, D, E):
             starts.append(starts[-1] + hi - lo)
         rows = starts[-1]
         parts = torch.full((rows, heads, slices, E), float("nan"), device=dev)
+        room = rows // chunk + 3 if chunk else 0
         ops.gla_scan(proj, off["q"], off["k"], off["v"], decay, q_scale, heads, D, E, state,
                      torch.tensor(starts + [0, 0], dtype=torch.int32, device=dev),
-                     torch.tensor(slots + [1], dtype=torch.int32, device=dev), 3, parts)
+                     torch.tensor(slots + [1], dtype=torch.int32, device=dev), 3, parts, chunk,
+                     torch.full((room, heads, D, E), float("nan"), device=dev) if chunk else None,
+                     torch.full((room, heads, D), float("nan"), device=dev) if chunk else None)
         out = torch.empty(rows, heads * E, dtype=dtype, device=dev)
         ops.gla_output(parts, heads, D, E, weight, eps, proj, off["g"], out)
         for i in range(3):
