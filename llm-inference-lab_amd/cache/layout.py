@@ -11,6 +11,10 @@ every wave instruction reads consecutive memory:
 (the same formulas as ``kcache_index`` / ``vcache_index`` in ``csrc/common.h``).
 The kernels never need this module; it serves tests, tools and anyone who wants
 to look into a cache from Python.
+
+The windowed attention with a sink keeps its keys row by row (``[..., P, D]``) and its
+values ``[..., P, E]`` in the order ``[P / 4][E][4]`` (the four keys of a quad side by side
+for each value channel): ``value_quads`` gives that view.
 """
 from __future__ import annotations
 
@@ -59,3 +63,10 @@ def values_to_cache_order(values: torch.Tensor) -> torch.Tensor:
 
 def values_from_cache_order(values: torch.Tensor) -> torch.Tensor:
     return _gather(values, value_index(values.shape[-1], values.shape[-2]))
+
+
+def value_quads(values: torch.Tensor) -> torch.Tensor:
+    """``[..., P, E]`` pages of the windowed attention's values as ``[..., P / 4, E, 4]``: entry
+    ``[..., o >> 2, e, o & 3]`` is channel ``e`` of the value of the key at offset ``o``."""
+    p, e = values.shape[-2], values.shape[-1]
+    return values.view(*values.shape[:-2], p // 4, e, 4)

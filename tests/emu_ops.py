@@ -272,8 +272,9 @@ class EmuOps:
         for r in range(rows):
             pos = int(positions[r])
             page = int(block_table[int(row_req[r]), pos // page_size])
-            k_cache[page, :, pos % page_size] = k[r]
-            v_cache[page, :, pos % page_size] = v[r]
+            o = pos % page_size
+            k_cache[page, :, o] = k[r]
+            cache_layout.value_quads(v_cache[page])[:, o >> 2, :, o & 3] = v[r]
 
     def sink_window_attention(self, q, num_heads, num_kv_heads, key_dim, value_dim, k_cache, v_cache, block_table,
                               page_size, positions, row_req, window, keep_first, sink, scale, out):
@@ -288,7 +289,7 @@ class EmuOps:
             pages = torch.tensor([int(block_table[b, j // page_size]) for j in js])
             offs = torch.tensor([j % page_size for j in js])
             k = k_cache[pages, :, offs].float()          # [keys, G, D]
-            v = v_cache[pages, :, offs].float()
+            v = cache_layout.value_quads(v_cache)[pages, :, offs >> 2, :, offs & 3].float()
             for h in range(num_heads):
                 s = (k[:, h // group] @ qf[r, h]) * scale
                 if sink is not None:

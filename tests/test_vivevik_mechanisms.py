@@ -8,6 +8,7 @@ import torch
 import helpers as H          # noqa: F401
 import plain_vivevik as P
 from emu_ops import EmuOps
+from llm_inference_lab_amd.cache.layout import value_quads
 
 BACKENDS = ["emu", pytest.param("hip", marks=pytest.mark.gpu)]
 DTYPES = [torch.float32, torch.bfloat16]
@@ -124,7 +125,7 @@ def test_norm_over_the_whole_projection_and_the_cache_write(backend, dtype):
     for pos in (0, 15, 16, 31, 36):
         page = int(cache.table[0, pos // 16])
         close(cache.k_cache[page, :, pos % 16], want_k[pos], dtype, f"key at {pos}")
-        close(cache.v_cache[page, :, pos % 16], want_v[pos], dtype, f"value at {pos}")
+        close(value_quads(cache.v_cache[page])[:, (pos % 16) >> 2, :, pos & 3], want_v[pos], dtype, f"value at {pos}")
     # a layer without keys and values of its own: queries only, the pages untouched
     before = cache.k_cache.clone()
     q2 = cache.write(proj[:, :H_ * D].contiguous(), H_, list(range(n)), [0] * n, qw, None, 1e-6, own_kv=False)
@@ -209,6 +210,46 @@ def test_attention_many_rows_at_once_and_the_sink(backend, dtype):
         close(out, want.reshape(n, -1), dtype, f"sink {sink_value}", f32=3e-5)
         if sink_value == 40.0:
             assert float(out.float().abs().max()) < 1e-6, "a sink that outweighs every key leaves nothing"
+
+
+@pytest.mark.parametrize("backend", BACKENDS)
+@pytest.mark.parametrize("H_,G,D,E", [(4, 2, 32, 16), (2, 1, 64, 48), (3, 3, 128, 128), (2, 2, 96, 80)])
+@pytest.mark.parametrize("window,keep_first", [(24, 3), (40, 20), (None, 0), (7, 0)])
+def test_attention_of_prompts_in_bfloat16_at_matrix_core_sizes(backend, H_, G, D, E, window, keep_first):
+    """Portions of three requests in one call (a history behind the first, tiles of 16 rows that
+    hold rows of two requests, a single decoded row), head sizes that the matrix-core kernel
+    takes; keys that stand out just inside and just outside the window and the kept prefix."""
+    ops = ops_of(backend)
+    dtype = torch.bfloat16
+    lengths = [120, 45, 70]                     # tokens each request has after the call
+    new = [50, 45, 1]                           # rows it brings to the call
+    ks = [randn(n, G, D, seed=30 + i) for i, n in enumerate(lengths)]
+    vs = [randn(n, G, E, seed=40 + i) for i, n in enumerate(lengths)]
+    qs = [randn(n, H_, D, seed=50 + i) for i, n in enumerate(lengths)]
+    w = window or 10 ** 6
+    stand_out = []
+    for b, n in enumerate(lengths):
+        for k_, (i, j) in enumerate([(n - 1, n - w), (n - 2, n - 1 - w), (n - 3, keep_first - 1), (n - 5, keep_first)]):
+            if 0 <= j <= i and i >= n - new[b] and j not in [x[2] for x in stand_out if x[0] == b]:
+                for h in range(H_):
+                    qs[b][i, h] = ks[b][j, h // (H_ // G)] * 6.0 / ks[b][j, h // (H_ // G)].norm()
+                stand_out.append((b, i, j))
+    cache = Paged(ops, dtype, lengths, G, D, E, seed=11)
+    for b, n in enumerate(lengths):             # everything into the pages (the history and the new rows)
+        proj = torch.cat([torch.zeros(n, H_ * D), ks[b].reshape(n, -1), vs[b].reshape(n, -1)], 1)
+        cache.write(proj, H_, list(range(n)), [b] * n)
+    rows_q = torch.cat([cache_rounded(qs[b][n - new[b]:], dtype) for b, n in enumerate(lengths)])
+    positions = [p for b, n in enumerate(lengths) for p in range(n - new[b], n)]
+    row_req = [b for b in range(3) for _ in range(new[b])]
+    sink = torch.tensor([0.5 * h - 0.3 for h in range(H_)]).to(ops.device)
+    out = cache.attend(rows_q.reshape(len(positions), -1).to(dtype).to(ops.device), H_, positions, row_req, window,
+                       keep_first, sink, 0.35)
+    at = 0
+    for b, n in enumerate(lengths):
+        want = P.sink_attention(cache_rounded(qs[b][n - new[b]:], dtype).to(F64), cache_rounded(ks[b], dtype).to(F64),
+                                cache_rounded(vs[b], dtype).to(F64), sink.cpu().to(F64), 0.35, w, keep_first)
+        close(out[at:at + new[b]], want.reshape(new[b], -1), dtype, f"request {b}", bf16=2.5e-2)
+        at += new[b]
 
 
 # ------------------------------------------------------------------ gated linear attention
