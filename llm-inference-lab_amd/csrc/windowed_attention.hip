@@ -155,7 +155,11 @@ __global__ __launch_bounds__(64) void sink_window_attention_kernel(
     const T* __restrict__ q, int n_heads, int n_kv, int D, int E, const T* __restrict__ k_cache,
     const T* __restrict__ v_cache, const int* __restrict__ table, int max_pages, int page_size,
     const int* __restrict__ positions, const int* __restrict__ row_req, int window, int keep_first,
-    const float* __restrict__ sink, float scale, T* __restrict__ out) {
+    const float* __restrict__ sink, float scale, T* __restrict__ out, const int* __restrict__ q_start, int long_from) {
+  if (long_from > 0) {      // (rows of requests that bring many rows are the other kernel's)
+    const int b = row_req[blockIdx.x];
+    if (q_start[b + 1] - q_start[b] >= long_from) return;
+  }
   extern __shared__ float lds[];       // q [D], weights [64], first value of each key's quad [64]
   float* qs = lds;
   float* ps = lds + D;
@@ -222,46 +226,151 @@ __global__ __launch_bounds__(64) void sink_window_attention_kernel(
   }
 }
 
-// ---- matrix-core kernel (bfloat16; D a multiple of 32, E of 16).  A wave takes 16
-// consecutive rows of the step and one head; a block four such tiles.  Keys come 32 at a
-// time as two blocks of 16 (each within a page).  The scores are taken transposed, S^T = K
-// Q^T, so that a lane ends up with the weights of ONE query for eight keys: exactly the
-// operand the second product O^T = V^T P^T wants, with no trip through LDS.  Lane l = 16 g +
-// c holds query c and, of a block of 16 keys, the keys 4 g .. 4 g + 3.  Rows of several
-// requests in one tile are served request after request (the others' columns masked).
+// ---- matrix-core kernels (bfloat16; D a multiple of 32, E of 16).  A wave serves 16 queries
+// that share their keys: 16 consecutive rows of the step for one head (prompts), or the
+// heads of one key/value head for one row (decoding: the keys are read once for the group).
+// Keys come 32 at a time as two blocks of 16 (each within a page).  The scores are taken
+// transposed, S^T = K Q^T, so that a lane ends up with the weights of ONE query for eight
+// keys: exactly the operand the second product O^T = V^T P^T wants, with no trip through
+// LDS.  Lane l = 16 g4 + c holds query c and, of a block of 16 keys, the keys 4 g4 .. 4 g4 + 3.
+template <int EB>
+struct Running {
+  float m, l;
+  floatx4 o[EB];
+};
+
+// The keys a wave's queries of one request can see, as a list of tiles of 32: first the kept
+// prefix [0, a_end), then [b_start, p_hi] (p_lo, p_hi: the lowest and highest position among
+// the queries; b_start: the lowest window's first key rounded down to 16).
+struct KeyTiles {
+  int a_end, b_start, end_b, tiles_a, tiles;
+  __device__ KeyTiles(int p_lo, int p_hi, int window, int keep_first) {
+    const int lo = window > 0 ? (p_lo - window + 1 > 0 ? p_lo - window + 1 : 0) : 0;
+    b_start = lo & ~15;
+    a_end = keep_first < b_start ? keep_first : b_start;
+    end_b = p_hi + 1;
+    tiles_a = (a_end + 31) >> 5;
+    tiles = tiles_a + ((end_b - b_start + 31) >> 5);
+  }
+};
+
+// Tiles [t_begin, t_end) of the list into the running softmax of the lane's query (position
+// pos; seen: whether this lane's query takes part at all).
 template <int DC, int EB>
-__global__ __launch_bounds__(256) void sink_window_attention_mfma_kernel(
-    const bf16_t* __restrict__ q, int n_rows, int n_heads, int n_kv, const bf16_t* __restrict__ k_cache,
-    const bf16_t* __restrict__ v_cache, const int* __restrict__ table, int max_pages, int page_size,
-    const int* __restrict__ positions, const int* __restrict__ row_req, int window, int keep_first,
-    const float* __restrict__ sink, float scale, bf16_t* __restrict__ out) {
+__device__ __forceinline__ void attend_tiles(const KeyTiles& kt, int t_begin, int t_end, const bf16x8 (&qf)[DC], bool seen,
+                                             int pos, const int* __restrict__ pages, int page_size, int n_kv, int g,
+                                             const bf16_t* __restrict__ k_cache, const bf16_t* __restrict__ v_cache,
+                                             int window, int keep_first, float scale, Running<EB>& run) {
+  constexpr int D = 32 * DC, E = 16 * EB;
+  const int lane = threadIdx.x & 63, c = lane & 15, g4 = lane >> 4;
+  for (int t = t_begin; t < t_end; ++t) {
+    const int j0 = t < kt.tiles_a ? 32 * t : kt.b_start + 32 * (t - kt.tiles_a);
+    const int end = t < kt.tiles_a ? kt.a_end : kt.end_b;
+    floatx4 s[2];
+    size_t vbase[2];
+    bool have[2];
+#pragma unroll
+    for (int u = 0; u < 2; ++u) {
+      const int ju = j0 + 16 * u;
+      have[u] = ju < end;
+      s[u] = floatx4{0.f, 0.f, 0.f, 0.f};
+      vbase[u] = 0;
+      if (have[u]) {
+        const int page = pages[ju / page_size];
+        const size_t head = ((size_t)page * n_kv + g) * page_size;
+        const int off = ju % page_size;
+        const bf16_t* kp = k_cache + (head + off + c) * D + 8 * g4;
+#pragma unroll
+        for (int dc = 0; dc < DC; ++dc)
+          s[u] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(*(const bf16x8*)(kp + 32 * dc), qf[dc], s[u], 0, 0, 0);
+        vbase[u] = head * E + (size_t)((off >> 2) + g4) * E * 4;
+      }
+    }
+    float tmax = NEG_INF;
+#pragma unroll
+    for (int u = 0; u < 2; ++u)
+#pragma unroll
+      for (int i = 0; i < 4; ++i) {
+        const int j = j0 + 16 * u + 4 * g4 + i;
+        const bool ok = have[u] && seen && j < end && sees(pos, j, window, keep_first);
+        s[u][i] = ok ? s[u][i] * scale : NEG_INF;
+        tmax = fmaxf(tmax, s[u][i]);
+      }
+    tmax = fmaxf(tmax, __shfl_xor(tmax, 16, WAVE));
+    tmax = fmaxf(tmax, __shfl_xor(tmax, 32, WAVE));
+    const float m_new = fmaxf(run.m, tmax);
+    const float m_use = m_new == NEG_INF ? 0.f : m_new;
+    const float corr = run.m == NEG_INF ? 0.f : __expf(run.m - m_use);
+    float sum = 0.f;
+    bf16x8 pf;
+#pragma unroll
+    for (int u = 0; u < 2; ++u)
+#pragma unroll
+      for (int i = 0; i < 4; ++i) {
+        const float p = __expf(s[u][i] - m_use);       // (exp(-inf) = 0 for a masked key)
+        sum += p;
+        pf[4 * u + i] = (bf16_t)p;
+      }
+    sum += __shfl_xor(sum, 16, WAVE);
+    sum += __shfl_xor(sum, 32, WAVE);
+    run.l = run.l * corr + sum;
+    run.m = m_new;
+#pragma unroll
+    for (int eb = 0; eb < EB; ++eb) {
+      bf16x8 vf;
+#pragma unroll
+      for (int u = 0; u < 2; ++u) {
+        bf16x4 quad = bf16x4{(bf16_t)0.f, (bf16_t)0.f, (bf16_t)0.f, (bf16_t)0.f};
+        if (have[u]) quad = *(const bf16x4*)(v_cache + vbase[u] + (size_t)(16 * eb + c) * 4);
+#pragma unroll
+        for (int i = 0; i < 4; ++i) vf[4 * u + i] = quad[i];
+      }
+#pragma unroll
+      for (int i = 0; i < 4; ++i) run.o[eb][i] *= corr;
+      run.o[eb] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(vf, pf, run.o[eb], 0, 0, 0);
+    }
+  }
+}
+
+struct MfmaArgs {
+  const bf16_t* q; int n_rows, n_heads, n_kv;
+  const bf16_t* k_cache; const bf16_t* v_cache; const int* table; int max_pages, page_size;
+  const int* positions; const int* row_req; int window, keep_first; const float* sink; float scale;
+  bf16_t* out; const int* q_start; int long_from;
+  int splits; float* part_o; float* part_ml;      // (decoding) [rows, heads, splits, E] and [rows, heads, splits, 2]
+};
+
+// Prompts: a wave takes 16 consecutive rows and one head, a block four such tiles.  Rows of
+// several requests in one tile are served request after request (the others' columns masked).
+template <int DC, int EB>
+__global__ __launch_bounds__(256) void sink_window_attention_mfma_kernel(MfmaArgs a) {
   constexpr int D = 32 * DC, E = 16 * EB;
   const int lane = threadIdx.x & 63, c = lane & 15, g4 = lane >> 4;
   const int r0 = (blockIdx.x * 4 + (threadIdx.x >> 6)) * 16;
-  if (r0 >= n_rows) return;
-  const int h = blockIdx.y, g = h / (n_heads / n_kv);
+  if (r0 >= a.n_rows) return;
+  const int h = blockIdx.y, g = h / (a.n_heads / a.n_kv);
   const int r = r0 + c;
-  const bool row_ok = r < n_rows;
-  const int pos = row_ok ? positions[r] : 0;
-  const int req = row_ok ? row_req[r] : -1;
+  const bool row_ok = r < a.n_rows;
+  const int pos = row_ok ? a.positions[r] : 0;
+  const int req = row_ok ? a.row_req[r] : -1;
   bf16x8 qf[DC];
 #pragma unroll
   for (int dc = 0; dc < DC; ++dc) {
-    if (row_ok) qf[dc] = *(const bf16x8*)(q + ((size_t)r * n_heads + h) * D + 32 * dc + 8 * g4);
+    if (row_ok) qf[dc] = *(const bf16x8*)(a.q + ((size_t)r * a.n_heads + h) * D + 32 * dc + 8 * g4);
     else
 #pragma unroll
-      for (int t = 0; t < 8; ++t) qf[dc][t] = (bf16_t)0.f;
+      for (int i = 0; i < 8; ++i) qf[dc][i] = (bf16_t)0.f;
   }
-  float m = sink ? sink[h] : NEG_INF;
-  float l = sink ? 1.f : 0.f;
-  floatx4 o[EB];
+  Running<EB> run;
+  run.m = a.sink ? a.sink[h] : NEG_INF;
+  run.l = a.sink ? 1.f : 0.f;
 #pragma unroll
-  for (int eb = 0; eb < EB; ++eb) o[eb] = floatx4{0.f, 0.f, 0.f, 0.f};
-  const int b_first = __builtin_amdgcn_readfirstlane(row_req[r0]);
-  const int b_last = __builtin_amdgcn_readfirstlane(row_req[(r0 + 15 < n_rows ? r0 + 15 : n_rows - 1)]);
+  for (int eb = 0; eb < EB; ++eb) run.o[eb] = floatx4{0.f, 0.f, 0.f, 0.f};
+  const int b_first = __builtin_amdgcn_readfirstlane(a.row_req[r0]);
+  const int b_last = __builtin_amdgcn_readfirstlane(a.row_req[(r0 + 15 < a.n_rows ? r0 + 15 : a.n_rows - 1)]);
   for (int b = b_first; b <= b_last; ++b) {
+    if (a.long_from > 0 && a.q_start[b + 1] - a.q_start[b] < a.long_from) continue;      // (the other kernels' rows)
     const bool mine = req == b;
-    // the first and the last position among this request's rows of the tile
     int p_lo = mine ? pos : 0x7fffffff, p_hi = mine ? pos : -1;
 #pragma unroll
     for (int off = 32; off > 0; off >>= 1) {
@@ -269,110 +378,117 @@ __global__ __launch_bounds__(256) void sink_window_attention_mfma_kernel(
       p_hi = max(p_hi, __shfl_xor(p_hi, off, WAVE));
     }
     if (p_hi < 0) continue;
-    const int lo = window > 0 ? (p_lo - window + 1 > 0 ? p_lo - window + 1 : 0) : 0;
-    const int b_start = lo & ~15;
-    const int a_end = keep_first < b_start ? keep_first : b_start;
-    const int* pages = table + (size_t)b * max_pages;
-    for (int run = 0; run < 2; ++run) {
-      const int first = run == 0 ? 0 : b_start;
-      const int end = run == 0 ? a_end : p_hi + 1;
-      for (int j0 = first; j0 < end; j0 += 32) {
-        floatx4 s[2];
-        size_t vbase[2];
-        bool have[2];
-#pragma unroll
-        for (int u = 0; u < 2; ++u) {
-          const int ju = j0 + 16 * u;
-          have[u] = ju < end;
-          s[u] = floatx4{0.f, 0.f, 0.f, 0.f};
-          vbase[u] = 0;
-          if (have[u]) {
-            const int page = pages[ju / page_size];
-            const size_t head = ((size_t)page * n_kv + g) * page_size;
-            const int off = ju % page_size;
-            const bf16_t* kp = k_cache + (head + off + c) * D + 8 * g4;
-#pragma unroll
-            for (int dc = 0; dc < DC; ++dc)
-              s[u] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(*(const bf16x8*)(kp + 32 * dc), qf[dc], s[u], 0, 0, 0);
-            vbase[u] = head * E + (size_t)((off >> 2) + g4) * E * 4;
-          }
-        }
-        float tmax = NEG_INF;
-#pragma unroll
-        for (int u = 0; u < 2; ++u)
-#pragma unroll
-          for (int t = 0; t < 4; ++t) {
-            const int j = j0 + 16 * u + 4 * g4 + t;
-            const bool ok = have[u] && mine && j < end && sees(pos, j, window, keep_first);
-            s[u][t] = ok ? s[u][t] * scale : NEG_INF;
-            tmax = fmaxf(tmax, s[u][t]);
-          }
-        tmax = fmaxf(tmax, __shfl_xor(tmax, 16, WAVE));
-        tmax = fmaxf(tmax, __shfl_xor(tmax, 32, WAVE));
-        const float m_new = fmaxf(m, tmax);
-        const float m_use = m_new == NEG_INF ? 0.f : m_new;
-        const float corr = m == NEG_INF ? 0.f : __expf(m - m_use);
-        float sum = 0.f;
-        bf16x8 pf;
-#pragma unroll
-        for (int u = 0; u < 2; ++u)
-#pragma unroll
-          for (int t = 0; t < 4; ++t) {
-            const float p = __expf(s[u][t] - m_use);       // (exp(-inf) = 0 for a masked key)
-            sum += p;
-            pf[4 * u + t] = (bf16_t)p;
-          }
-        sum += __shfl_xor(sum, 16, WAVE);
-        sum += __shfl_xor(sum, 32, WAVE);
-        l = l * corr + sum;
-        m = m_new;
-#pragma unroll
-        for (int eb = 0; eb < EB; ++eb) {
-          bf16x8 vf;
-#pragma unroll
-          for (int u = 0; u < 2; ++u) {
-            bf16x4 quad = bf16x4{(bf16_t)0.f, (bf16_t)0.f, (bf16_t)0.f, (bf16_t)0.f};
-            if (have[u]) quad = *(const bf16x4*)(v_cache + vbase[u] + (size_t)(16 * eb + c) * 4);
-#pragma unroll
-            for (int t = 0; t < 4; ++t) vf[4 * u + t] = quad[t];
-          }
-#pragma unroll
-          for (int t = 0; t < 4; ++t) o[eb][t] *= corr;
-          o[eb] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(vf, pf, o[eb], 0, 0, 0);
-        }
-      }
-    }
+    const KeyTiles kt(p_lo, p_hi, a.window, a.keep_first);
+    attend_tiles<DC, EB>(kt, 0, kt.tiles, qf, mine, pos, a.table + (size_t)b * a.max_pages, a.page_size, a.n_kv, g,
+                         a.k_cache, a.v_cache, a.window, a.keep_first, a.scale, run);
   }
   if (!row_ok) return;
-  const float inv = 1.0f / l;
+  if (a.long_from > 0 && a.q_start[req + 1] - a.q_start[req] < a.long_from) return;
+  const float inv = 1.0f / run.l;
 #pragma unroll
   for (int eb = 0; eb < EB; ++eb) {
     bf16x4 w;
 #pragma unroll
-    for (int t = 0; t < 4; ++t) w[t] = (bf16_t)(o[eb][t] * inv);
-    *(bf16x4*)(out + ((size_t)r * n_heads + h) * E + 16 * eb + 4 * g4) = w;
+    for (int i = 0; i < 4; ++i) w[i] = (bf16_t)(run.o[eb][i] * inv);
+    *(bf16x4*)(a.out + ((size_t)r * a.n_heads + h) * E + 16 * eb + 4 * g4) = w;
+  }
+}
+
+// Decoding (requests that bring fewer than long_from rows): a wave takes ONE row, the heads of
+// one key/value head (16 at a time) and one of `splits` shares of the row's key tiles, so that
+// few rows still fill the chip.  With one share the result is final; else the share's
+// maximum, denominator and unnormalised sum go to part_ml / part_o for the merge kernel.
+// The sink enters the first share only.
+template <int DC, int EB>
+__global__ __launch_bounds__(64) void sink_window_attention_grouped_kernel(MfmaArgs a) {
+  constexpr int D = 32 * DC, E = 16 * EB;
+  const int lane = threadIdx.x & 63, c = lane & 15, g4 = lane >> 4;
+  const int r = blockIdx.x;
+  const int b = a.row_req[r];
+  if (a.long_from > 0 && a.q_start[b + 1] - a.q_start[b] >= a.long_from) return;      // (the prompts' kernel's rows)
+  const int group = a.n_heads / a.n_kv, per_group = (group + 15) >> 4;
+  const int g = blockIdx.y / per_group;
+  const int hc = (blockIdx.y % per_group) * 16 + c;        // this lane's head within the group
+  const bool head_ok = hc < group;
+  const int h = g * group + hc;
+  const int pos = a.positions[r];
+  bf16x8 qf[DC];
+#pragma unroll
+  for (int dc = 0; dc < DC; ++dc) {
+    if (head_ok) qf[dc] = *(const bf16x8*)(a.q + ((size_t)r * a.n_heads + h) * D + 32 * dc + 8 * g4);
+    else
+#pragma unroll
+      for (int i = 0; i < 8; ++i) qf[dc][i] = (bf16_t)0.f;
+  }
+  const int z = blockIdx.z;
+  Running<EB> run;
+  run.m = (a.sink && head_ok && z == 0) ? a.sink[h] : NEG_INF;
+  run.l = (a.sink && head_ok && z == 0) ? 1.f : 0.f;
+#pragma unroll
+  for (int eb = 0; eb < EB; ++eb) run.o[eb] = floatx4{0.f, 0.f, 0.f, 0.f};
+  const KeyTiles kt(pos, pos, a.window, a.keep_first);
+  const int per = (kt.tiles + a.splits - 1) / a.splits;
+  const int t_begin = z * per, t_end = (z + 1) * per < kt.tiles ? (z + 1) * per : kt.tiles;
+  attend_tiles<DC, EB>(kt, t_begin, t_end, qf, head_ok, pos, a.table + (size_t)b * a.max_pages, a.page_size, a.n_kv, g,
+                       a.k_cache, a.v_cache, a.window, a.keep_first, a.scale, run);
+  if (!head_ok) return;
+  if (a.splits == 1) {
+    const float inv = 1.0f / run.l;
+#pragma unroll
+    for (int eb = 0; eb < EB; ++eb) {
+      bf16x4 w;
+#pragma unroll
+      for (int i = 0; i < 4; ++i) w[i] = (bf16_t)(run.o[eb][i] * inv);
+      *(bf16x4*)(a.out + ((size_t)r * a.n_heads + h) * E + 16 * eb + 4 * g4) = w;
+    }
+    return;
+  }
+  const size_t share = ((size_t)r * a.n_heads + h) * a.splits + z;
+  if (g4 == 0) {
+    a.part_ml[share * 2] = run.m;
+    a.part_ml[share * 2 + 1] = run.l;
+  }
+#pragma unroll
+  for (int eb = 0; eb < EB; ++eb) *(floatx4*)(a.part_o + share * E + 16 * eb + 4 * g4) = run.o[eb];
+}
+
+// out[r, h] = sum_z exp(m_z - M) o_z / sum_z exp(m_z - M) l_z over the shares of the row's keys.
+__global__ __launch_bounds__(64) void sink_window_attention_merge_kernel(MfmaArgs a, int E) {
+  const int r = blockIdx.x, h = blockIdx.y;
+  const int b = a.row_req[r];
+  if (a.long_from > 0 && a.q_start[b + 1] - a.q_start[b] >= a.long_from) return;
+  const size_t first = ((size_t)r * a.n_heads + h) * a.splits;
+  float big = NEG_INF;
+  for (int z = 0; z < a.splits; ++z) big = fmaxf(big, a.part_ml[(first + z) * 2]);
+  float den = 0.f;
+  for (int z = 0; z < a.splits; ++z) {
+    const float m = a.part_ml[(first + z) * 2];
+    if (m != NEG_INF) den += __expf(m - big) * a.part_ml[(first + z) * 2 + 1];
+  }
+  for (int e = threadIdx.x; e < E; e += 64) {
+    float acc = 0.f;
+    for (int z = 0; z < a.splits; ++z) {
+      const float m = a.part_ml[(first + z) * 2];
+      if (m != NEG_INF) acc = fmaf(__expf(m - big), a.part_o[(first + z) * E + e], acc);
+    }
+    a.out[((size_t)r * a.n_heads + h) * E + e] = (bf16_t)(acc / den);
   }
 }
 
 static int g_force_plain = 0;
 extern "C" void llmlab_debug_windowed_attention_plain(int on) { g_force_plain = on; }
 
-// Whether a call of these sizes goes to the matrix-core kernel.
-extern "C" int llmlab_sink_window_attention_uses_mfma(int dtype, int rows, int D, int E, int page_size) {
-  return !g_force_plain && dtype == DT_BF16 && rows >= 32 && D % 32 == 0 && D <= 128 && E % 16 == 0 && E <= 128 &&
-         page_size % 16 == 0;
+// Whether the matrix-core kernel takes these sizes at all.
+extern "C" int llmlab_sink_window_attention_has_mfma(int dtype, int D, int E, int page_size) {
+  return !g_force_plain && dtype == DT_BF16 && D % 32 == 0 && D <= 128 && E % 16 == 0 && E <= 128 && page_size % 16 == 0;
 }
 
 template <int DC>
-static void launch_mfma(int EBv, dim3 grid, hipStream_t stream, const bf16_t* q, int rows, int n_heads, int n_kv,
-                        const bf16_t* k_cache, const bf16_t* v_cache, const int* table, int max_pages, int page_size,
-                        const int* positions, const int* row_req, int window, int keep_first, const float* sink,
-                        float scale, bf16_t* out) {
-#define LLMLAB_MFMA(EBC)                                                                                          \
-  case EBC:                                                                                                       \
-    hipLaunchKernelGGL((sink_window_attention_mfma_kernel<DC, EBC>), grid, dim3(256), 0, stream, q, rows, n_heads, \
-                       n_kv, k_cache, v_cache, table, max_pages, page_size, positions, row_req, window, keep_first, \
-                       sink, scale, out);                                                                         \
+static void launch_mfma(int EBv, int which, dim3 grid, dim3 block, hipStream_t stream, const MfmaArgs& a) {
+#define LLMLAB_MFMA(EBC)                                                                                      \
+  case EBC:                                                                                                   \
+    if (which == 0) hipLaunchKernelGGL((sink_window_attention_mfma_kernel<DC, EBC>), grid, block, 0, stream, a); \
+    else hipLaunchKernelGGL((sink_window_attention_grouped_kernel<DC, EBC>), grid, block, 0, stream, a);      \
     break;
   switch (EBv) {
     LLMLAB_MFMA(1) LLMLAB_MFMA(2) LLMLAB_MFMA(3) LLMLAB_MFMA(4) LLMLAB_MFMA(5) LLMLAB_MFMA(6) LLMLAB_MFMA(7) LLMLAB_MFMA(8)
@@ -380,12 +496,28 @@ static void launch_mfma(int EBv, dim3 grid, hipStream_t stream, const bf16_t* q,
 #undef LLMLAB_MFMA
 }
 
+static void launch_mfma_any(int D, int E, int which, dim3 grid, dim3 block, hipStream_t stream, const MfmaArgs& a) {
+  switch (D / 32) {
+    case 1: launch_mfma<1>(E / 16, which, grid, block, stream, a); break;
+    case 2: launch_mfma<2>(E / 16, which, grid, block, stream, a); break;
+    case 3: launch_mfma<3>(E / 16, which, grid, block, stream, a); break;
+    default: launch_mfma<4>(E / 16, which, grid, block, stream, a); break;
+  }
+}
+
 // q [rows, heads * D], out [rows, heads * E] in the compute dtype; sink: float32 [heads] or null.
 // The rows of a request are adjacent and requests come in rising order of row_req.
+// long_from > 0 (sizes that the matrix-core kernels take only): requests that bring at least so
+// many rows (q_start[b + 1] - q_start[b]) go to the prompts' kernel, the others to the decoding
+// one; `launches` says which of the two the step needs (bit 0 decoding, bit 1 prompts).
+// max_keys: the most keys a decoding row of this step sees (it sets how many shares a row's
+// keys are cut into); workspace: float32 scratch for the shares' partial results.
 extern "C" int llmlab_sink_window_attention(const void* q, int dtype, int rows, int n_heads, int n_kv, int D, int E,
                                             const void* k_cache, const void* v_cache, const int* table, int max_pages,
                                             int page_size, const int* positions, const int* row_req, int window,
                                             int keep_first, const float* sink, float scale, void* out,
+                                            const int* q_start, int long_from, int launches, int max_keys,
+                                            float* workspace, size_t workspace_floats, int num_cus,
                                             hipStream_t stream) {
   LLMLAB_REQUIRE(rows >= 0 && n_heads > 0 && n_kv > 0 && n_heads % n_kv == 0 && D > 0 && E > 0,
                  "sink_window_attention: bad sizes rows=%d heads=%d kv=%d D=%d E=%d", rows, n_heads, n_kv, D, E);
@@ -394,19 +526,43 @@ extern "C" int llmlab_sink_window_attention(const void* q, int dtype, int rows, 
   LLMLAB_REQUIRE(keep_first >= 0 && page_size > 0 && page_size % 4 == 0 && max_pages > 0,
                  "sink_window_attention: bad window or page arguments");
   if (rows == 0) return 0;
-  if (llmlab_sink_window_attention_uses_mfma(dtype, rows, D, E, page_size)) {
-    dim3 grid((rows + 63) / 64, n_heads);
-#define LLMLAB_ARGS E / 16, grid, stream, (const bf16_t*)q, rows, n_heads, n_kv, (const bf16_t*)k_cache,             \
-                    (const bf16_t*)v_cache, table, max_pages, page_size, positions, row_req, window, keep_first, sink, \
-                    scale, (bf16_t*)out
-    switch (D / 32) {
-      case 1: launch_mfma<1>(LLMLAB_ARGS); break;
-      case 2: launch_mfma<2>(LLMLAB_ARGS); break;
-      case 3: launch_mfma<3>(LLMLAB_ARGS); break;
-      default: launch_mfma<4>(LLMLAB_ARGS); break;
+  if (long_from > 0) {
+    LLMLAB_REQUIRE(q_start != nullptr && llmlab_sink_window_attention_has_mfma(dtype, D, E, page_size) && (launches & 3),
+                   "sink_window_attention: the matrix-core kernel does not take these sizes (D=%d E=%d page=%d)", D, E,
+                   page_size);
+  }
+  if (long_from > 0) {
+    MfmaArgs a{(const bf16_t*)q, rows, n_heads, n_kv, (const bf16_t*)k_cache, (const bf16_t*)v_cache, table, max_pages,
+               page_size, positions, row_req, window, keep_first, sink, scale, (bf16_t*)out, q_start, long_from, 1,
+               nullptr, nullptr};
+    if (launches & 2) {
+      launch_mfma_any(D, E, 0, dim3((rows + 63) / 64, n_heads), dim3(256), stream, a);
+      LLMLAB_LAUNCH_CHECK("sink_window_attention (prompts)");
     }
-#undef LLMLAB_ARGS
-    LLMLAB_LAUNCH_CHECK("sink_window_attention (matrix cores)");
+    if (launches & 1) {
+      // shares of a row's keys: enough waves for every compute unit a few times, a share no
+      // shorter than two tiles of 32 keys, and no more than the scratch holds
+      const int group = n_heads / n_kv, per_group = (group + 15) / 16;
+      const long waves = (long)rows * n_kv * per_group;
+      const int tiles = (max_keys + 31) / 32 + 1;
+      long splits = (4L * num_cus + waves - 1) / waves;
+      if (splits > tiles / 2) splits = tiles / 2;
+      const size_t per_split = (size_t)rows * n_heads * (E + 2);
+      if (workspace == nullptr) splits = 1;
+      else if (splits * per_split > workspace_floats) splits = (long)(workspace_floats / per_split);
+      if (splits < 1) splits = 1;
+      if (splits > 65535) splits = 65535;
+      a.splits = (int)splits;
+      a.part_o = workspace;
+      a.part_ml = workspace ? workspace + (size_t)rows * n_heads * splits * E : nullptr;
+      LLMLAB_REQUIRE(n_kv * per_group <= 65535, "sink_window_attention: too many heads");
+      launch_mfma_any(D, E, 1, dim3(rows, n_kv * per_group, a.splits), dim3(64), stream, a);
+      LLMLAB_LAUNCH_CHECK("sink_window_attention (decoding)");
+      if (a.splits > 1) {
+        hipLaunchKernelGGL(sink_window_attention_merge_kernel, dim3(rows, n_heads), dim3(64), 0, stream, a, E);
+        LLMLAB_LAUNCH_CHECK("sink_window_attention (merge)");
+      }
+    }
     return 0;
   }
   const size_t lds = (size_t)(D + 64 + (D & 1)) * sizeof(float) + 64 * sizeof(size_t);
@@ -414,11 +570,11 @@ extern "C" int llmlab_sink_window_attention(const void* q, int dtype, int rows, 
   if (dtype == DT_BF16)
     hipLaunchKernelGGL(sink_window_attention_kernel<bf16_t>, grid, block, lds, stream, (const bf16_t*)q, n_heads, n_kv, D,
                        E, (const bf16_t*)k_cache, (const bf16_t*)v_cache, table, max_pages, page_size, positions,
-                       row_req, window, keep_first, sink, scale, (bf16_t*)out);
+                       row_req, window, keep_first, sink, scale, (bf16_t*)out, q_start, long_from);
   else
     hipLaunchKernelGGL(sink_window_attention_kernel<float>, grid, block, lds, stream, (const float*)q, n_heads, n_kv, D,
                        E, (const float*)k_cache, (const float*)v_cache, table, max_pages, page_size, positions,
-                       row_req, window, keep_first, sink, scale, (float*)out);
+                       row_req, window, keep_first, sink, scale, (float*)out, q_start, long_from);
   LLMLAB_LAUNCH_CHECK("sink_window_attention");
   return 0;
 }

@@ -69,6 +69,11 @@ class DispatchRules:
     # 2,048 rows, 7 heads of 64 x 128: 1.53 ms in one run.
     scan_min_chunk: int = 16
     scan_max_chunk: int = 64
+    # Windowed attention with a sink: a request that brings at least this many rows to a step is
+    # served by the matrix-core kernel (tiles of 16 rows of one request), the others row by row
+    # by the plain kernel.  64 decoding requests in tiles of 16 rows of 16 requests: 14.3 ms a
+    # step against 1.9.
+    windowed_attention_long_rows: int = 4
     # Debug only: a product that the tiled kernel cuts gets this many pieces whatever the
     # estimate says (0: the estimate decides).
     forced_tiled_pieces: int = 0

@@ -991,8 +991,13 @@ class HipOps:
                 lib.llmlab_project_norm_write.restype = _c_int
                 lib.llmlab_sink_window_attention.argtypes = [
                     _c_ptr, _c_int, _c_int, _c_int, _c_int, _c_int, _c_int, _c_ptr, _c_ptr, _c_ptr, _c_int, _c_int,
-                    _c_ptr, _c_ptr, _c_int, _c_int, _c_ptr, _c_float, _c_ptr, _c_ptr]
+                    _c_ptr, _c_ptr, _c_int, _c_int, _c_ptr, _c_float, _c_ptr, _c_ptr, _c_int, _c_int, _c_int, _c_ptr,
+                    _c_size, _c_int, _c_ptr]
                 lib.llmlab_sink_window_attention.restype = _c_int
+                lib.llmlab_sink_window_attention_has_mfma.argtypes = [_c_int, _c_int, _c_int, _c_int]
+                lib.llmlab_sink_window_attention_has_mfma.restype = _c_int
+                lib.llmlab_debug_windowed_attention_plain.argtypes = [_c_int]
+                lib.llmlab_debug_windowed_attention_plain.restype = None
             elif kind == "linear_attention":
                 lib.llmlab_gla_decay.argtypes = [_c_ptr, _c_int, _c_int, _c_int, _c_ptr, _c_ptr, _c_float, _c_ptr,
                                                  _c_int, _c_ptr]
@@ -1071,12 +1076,34 @@ class HipOps:
                    self._ptr(block_table) if own_kv else None, block_table.stride(0) if own_kv else 0,
                    self._stream(), lib=lib)
 
+    def windowed_attention_long_rows(self, dtype, key_dim: int, value_dim: int, page_size: int) -> int:
+        """From how many rows on a request's share of a step goes to the matrix-core kernel of the
+        windowed attention (0: these sizes have none, every row goes to the plain kernel)."""
+        lib = self._mixer_lib("windowed_attention")
+        dt = DT_BF16 if dtype == torch.bfloat16 else DT_F32
+        if not lib.llmlab_sink_window_attention_has_mfma(dt, int(key_dim), int(value_dim), int(page_size)):
+            return 0
+        return int(self.rules.windowed_attention_long_rows)
+
+    def force_plain_windowed_attention(self, on: bool) -> None:
+        """Tests and measurements: no matrix-core kernel for the windowed attention."""
+        self._mixer_lib("windowed_attention").llmlab_debug_windowed_attention_plain(1 if on else 0)
+        self.debug_epoch += 1
+
     def sink_window_attention(self, q, num_heads, num_kv_heads, key_dim, value_dim, k_cache, v_cache, block_table,
-                              page_size, positions, row_req, window, keep_first, sink, scale, out) -> None:
+                              page_size, positions, row_req, window, keep_first, sink, scale, out,
+                              q_start=None, long_from=0, launches=3, max_keys=0) -> None:
         """The query of row ``r`` at position ``i = positions[r]`` of request ``row_req[r]`` attends
         to the cached keys ``j <= i`` with ``i - j < window`` or ``j < keep_first`` (``window`` None:
-        all); ``sink`` (float32 per head, or None) adds ``exp(sink)`` to the softmax's denominator."""
+        all); ``sink`` (float32 per head, or None) adds ``exp(sink)`` to the softmax's denominator.
+        ``long_from > 0`` (``windowed_attention_long_rows``: sizes that the matrix cores take):
+        requests that bring at least so many rows (by ``q_start``) are served in tiles of 16 rows
+        of a head, the others a row and a group of heads at a time with the row's keys cut into
+        shares; ``launches``: which of the two this step needs (bit 0 few rows, bit 1 many);
+        ``max_keys``: the most keys a row of this step sees (sets the number of shares)."""
         lib = self._mixer_lib("windowed_attention")
+        if long_from:
+            self._need(q_start, "request row starts", torch.int32)
         self._need(q, "queries")
         self._need(out, "attention output")
         rows = q.shape[0]
@@ -1102,7 +1129,9 @@ class HipOps:
         self._call(lib.llmlab_sink_window_attention, self._ptr(q), _dt(q), rows, num_heads, num_kv_heads, key_dim,
                    value_dim, self._ptr(k_cache), self._ptr(v_cache), self._ptr(block_table), block_table.stride(0),
                    page_size, self._ptr(positions), self._ptr(row_req), int(window) if window else 0,
-                   int(keep_first or 0), self._ptr(sink), float(scale), self._ptr(out), self._stream(), lib=lib)
+                   int(keep_first or 0), self._ptr(sink), float(scale), self._ptr(out),
+                   self._ptr(q_start) if long_from else None, int(long_from), int(launches), int(max_keys),
+                   self._ptr(self.workspace), self.workspace.numel(), self.num_cus, self._stream(), lib=lib)
 
     def gla_slices(self, key_dim: int) -> int:
         """Into how many pieces the scan leaves each output (one per slice of key channels)."""

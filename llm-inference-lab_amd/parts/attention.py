@@ -322,9 +322,22 @@ class WindowedSinkAttention(Mixer):
                                self.q_norm, self.k_norm, self.norm_eps, q, entry.k_cache, entry.v_cache,
                                group.page_size, ctx.positions, ctx.row_req, group.block_table)
         mixed = ctx.scratch("windowed_attention.out", (rows, self.num_heads * self.value_dim), self.dtype)
-        ops.sink_window_attention(q, self.num_heads, self.num_kv_heads, self.key_dim, self.value_dim, entry.k_cache,
-                                  entry.v_cache, group.block_table, group.page_size, ctx.positions, ctx.row_req,
-                                  self.window, self.keep_first, self.sink, self.scale, mixed)
+
+        def attend():
+            # (which requests bring many rows is read from the step's description when the launch
+            # is made, also when it is made again from a kept sequence of calls)
+            long_from, launches = self._split(ctx, group.page_size)
+            ops.sink_window_attention(q, self.num_heads, self.num_kv_heads, self.key_dim, self.value_dim,
+                                      entry.k_cache, entry.v_cache, group.block_table, group.page_size,
+                                      ctx.positions, ctx.row_req, self.window, self.keep_first, self.sink,
+                                      self.scale, mixed, ctx.all_q_start, long_from, launches,
+                                      ctx.max_ctx_len if self.window is None
+                                      else min(ctx.max_ctx_len, self.window + self.keep_first))
+        live = getattr(ops, "live", None)
+        if live is not None:
+            live(attend)
+        else:
+            attend()
         ops.linear_logits(mixed, self.w_o, out)
 
     def forward(self, h, residual, ctx, entry):
@@ -334,7 +347,22 @@ class WindowedSinkAttention(Mixer):
         self.forward_into(h, y[0], ctx, entry)
         self.ops.add_pending(residual, PendingSums(y, 1))
 
-    keeps_launches = True      # (every argument is a buffer of the step or a size of the layer)
+    def _split(self, ctx, page_size):
+        """``(long_from, launches)`` of this step: requests of at least ``long_from`` rows go to the
+        matrix-core kernel; worked out once per step, kept in the step's notes for the other layers."""
+        pick = getattr(self.ops, "windowed_attention_long_rows", None)
+        long_from = pick(self.dtype, self.key_dim, self.value_dim, page_size) if pick is not None else 0
+        if not long_from:
+            return 0, 1
+        key = ("windowed_attention.split", long_from)
+        if key not in ctx.memo:
+            starts = ctx.host_q_start
+            counts = [starts[b + 1] - starts[b] for b in range(ctx.n_reqs)]
+            ctx.memo[key] = ((1 if any(n < long_from for n in counts) else 0)
+                             | (2 if any(n >= long_from for n in counts) else 0))
+        return long_from, ctx.memo[key]
+
+    keeps_launches = True      # (what depends on the step beyond its rows is asked for at the launch)
 
     def kernel_libraries(self):
         return [("windowed_attention", None)]

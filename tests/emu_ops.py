@@ -277,7 +277,9 @@ class EmuOps:
             cache_layout.value_quads(v_cache[page])[:, o >> 2, :, o & 3] = v[r]
 
     def sink_window_attention(self, q, num_heads, num_kv_heads, key_dim, value_dim, k_cache, v_cache, block_table,
-                              page_size, positions, row_req, window, keep_first, sink, scale, out):
+                              page_size, positions, row_req, window, keep_first, sink, scale, out,
+                              q_start=None, long_from=0, launches=3, max_keys=0):
+        """(``long_from``, ``launches``: how the kernels share the rows; the result is the same.)"""
         self._count("sink_window_attention")
         rows = q.shape[0]
         qf = q.float().view(rows, num_heads, key_dim)

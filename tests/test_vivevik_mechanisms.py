@@ -98,11 +98,19 @@ class Paged:
 
     def attend(self, q, heads, positions, row_req, window, keep_first, sink, scale):
         dev = self.ops.device
-        out = torch.empty(q.shape[0], heads * self.E, dtype=self.dtype, device=dev)
+        out = torch.full((q.shape[0], heads * self.E), float("nan"), dtype=self.dtype, device=dev)
+        # as the attention part does: requests that bring many rows go to the matrix-core kernel
+        # where the sizes have one, the others to the plain kernel
+        pick = getattr(self.ops, "windowed_attention_long_rows", None)
+        long_from = pick(self.dtype, self.D, self.E, self.page) if pick is not None else 0
+        counts = [row_req.count(b) for b in range(max(row_req) + 1)]
+        starts = [sum(counts[:b]) for b in range(len(counts) + 1)]
+        launches = (1 if any(n < long_from for n in counts if n) else 0) | (2 if any(n >= long_from for n in counts) else 0)
         self.ops.sink_window_attention(q, heads, self.G, self.D, self.E, self.k_cache, self.v_cache, self.table,
                                        self.page, torch.tensor(positions, dtype=torch.int32, device=dev),
                                        torch.tensor(row_req, dtype=torch.int32, device=dev), window, keep_first,
-                                       sink, scale, out)
+                                       sink, scale, out, torch.tensor(starts, dtype=torch.int32, device=dev),
+                                       long_from, launches if long_from else 1, max(positions) + 1)
         return out
 
 
@@ -242,6 +250,44 @@ def test_attention_of_prompts_in_bfloat16_at_matrix_core_sizes(backend, H_, G, D
     positions = [p for b, n in enumerate(lengths) for p in range(n - new[b], n)]
     row_req = [b for b in range(3) for _ in range(new[b])]
     sink = torch.tensor([0.5 * h - 0.3 for h in range(H_)]).to(ops.device)
+    out = cache.attend(rows_q.reshape(len(positions), -1).to(dtype).to(ops.device), H_, positions, row_req, window,
+                       keep_first, sink, 0.35)
+    at = 0
+    for b, n in enumerate(lengths):
+        want = P.sink_attention(cache_rounded(qs[b][n - new[b]:], dtype).to(F64), cache_rounded(ks[b], dtype).to(F64),
+                                cache_rounded(vs[b], dtype).to(F64), sink.cpu().to(F64), 0.35, w, keep_first)
+        close(out[at:at + new[b]], want.reshape(new[b], -1), dtype, f"request {b}", bf16=2.5e-2)
+        at += new[b]
+
+
+@pytest.mark.parametrize("backend", BACKENDS)
+@pytest.mark.parametrize("H_,G,D,E", [(14, 2, 64, 64), (4, 4, 32, 16), (40, 2, 32, 32)])
+@pytest.mark.parametrize("window,keep_first", [(100, 4), (None, 0), (33, 40)])
+def test_attention_of_decoding_rows_in_bfloat16_at_matrix_core_sizes(backend, H_, G, D, E, window, keep_first):
+    """One row each of several requests with histories of different lengths (the keys of a row
+    are cut into shares that are merged afterwards; groups of 7, 1 and 20 heads per key/value
+    head), beside a request of three rows; a key that stands out at the window's edge."""
+    ops = ops_of(backend)
+    dtype = torch.bfloat16
+    lengths = [300, 1, 17, 131, 64]
+    new = [1, 1, 3, 1, 1]
+    ks = [randn(n, G, D, seed=60 + i) for i, n in enumerate(lengths)]
+    vs = [randn(n, G, E, seed=70 + i) for i, n in enumerate(lengths)]
+    qs = [randn(n, H_, D, seed=80 + i) for i, n in enumerate(lengths)]
+    w = window or 10 ** 6
+    for b, n in enumerate(lengths):
+        j = n - w if b % 2 == 0 else n - w - 1           # just inside / just outside the last row's window
+        if 0 <= j < n:
+            for h in range(H_):
+                qs[b][n - 1, h] = ks[b][j, h // (H_ // G)] * 6.0 / ks[b][j, h // (H_ // G)].norm()
+    cache = Paged(ops, dtype, lengths, G, D, E, seed=12)
+    for b, n in enumerate(lengths):
+        proj = torch.cat([torch.zeros(n, H_ * D), ks[b].reshape(n, -1), vs[b].reshape(n, -1)], 1)
+        cache.write(proj, H_, list(range(n)), [b] * n)
+    rows_q = torch.cat([cache_rounded(qs[b][n - new[b]:], dtype) for b, n in enumerate(lengths)])
+    positions = [p for b, n in enumerate(lengths) for p in range(n - new[b], n)]
+    row_req = [b for b in range(len(lengths)) for _ in range(new[b])]
+    sink = torch.tensor([0.1 * h - 0.5 for h in range(H_)]).to(ops.device)
     out = cache.attend(rows_q.reshape(len(positions), -1).to(dtype).to(ops.device), H_, positions, row_req, window,
                        keep_first, sink, 0.35)
     at = 0
