@@ -254,45 +254,86 @@ struct KeyTiles {
   }
 };
 
+// What a wave holds of one tile of 32 keys before the products: the keys' fragments of both
+// blocks of 16, where the blocks' values start, and the tile's place.
+template <int DC>
+struct KeyFrags {
+  bf16x8 k[2][DC];
+  size_t vbase[2];
+  bool have[2];
+  int j0, end;
+};
+
+template <int DC, int E>
+__device__ __forceinline__ void load_keys(KeyFrags<DC>& f, const KeyTiles& kt, int t, const int* __restrict__ pages,
+                                          int page_size, int n_kv, int g, const bf16_t* __restrict__ k_cache) {
+  constexpr int D = 32 * DC;
+  const int lane = threadIdx.x & 63, c = lane & 15, g4 = lane >> 4;
+  f.j0 = t < kt.tiles_a ? 32 * t : kt.b_start + 32 * (t - kt.tiles_a);
+  f.end = t < kt.tiles_a ? kt.a_end : kt.end_b;
+#pragma unroll
+  for (int u = 0; u < 2; ++u) {
+    const int ju = f.j0 + 16 * u;
+    f.have[u] = ju < f.end;
+    f.vbase[u] = 0;
+    if (f.have[u]) {
+      const int page = pages[ju / page_size];
+      const size_t head = ((size_t)page * n_kv + g) * page_size;
+      const int off = ju % page_size;
+      const bf16_t* kp = k_cache + (head + off + c) * D + 8 * g4;
+#pragma unroll
+      for (int dc = 0; dc < DC; ++dc) f.k[u][dc] = *(const bf16x8*)(kp + 32 * dc);
+      f.vbase[u] = head * E + (size_t)((off >> 2) + g4) * E * 4;
+    } else {
+#pragma unroll
+      for (int dc = 0; dc < DC; ++dc)
+#pragma unroll
+        for (int i = 0; i < 8; ++i) f.k[u][dc][i] = (bf16_t)0.f;
+    }
+  }
+}
+
 // Tiles [t_begin, t_end) of the list into the running softmax of the lane's query (position
-// pos; seen: whether this lane's query takes part at all).
+// pos; seen: whether this lane's query takes part at all).  The loads run ahead of the
+// products: a tile's values are asked for before its scores are taken, the next tile's keys
+// before this tile's softmax.
 template <int DC, int EB>
 __device__ __forceinline__ void attend_tiles(const KeyTiles& kt, int t_begin, int t_end, const bf16x8 (&qf)[DC], bool seen,
                                              int pos, const int* __restrict__ pages, int page_size, int n_kv, int g,
                                              const bf16_t* __restrict__ k_cache, const bf16_t* __restrict__ v_cache,
                                              int window, int keep_first, float scale, Running<EB>& run) {
-  constexpr int D = 32 * DC, E = 16 * EB;
+  constexpr int E = 16 * EB;
   const int lane = threadIdx.x & 63, c = lane & 15, g4 = lane >> 4;
+  if (t_begin >= t_end) return;
+  KeyFrags<DC> cur, nxt;
+  load_keys<DC, E>(cur, kt, t_begin, pages, page_size, n_kv, g, k_cache);
   for (int t = t_begin; t < t_end; ++t) {
-    const int j0 = t < kt.tiles_a ? 32 * t : kt.b_start + 32 * (t - kt.tiles_a);
-    const int end = t < kt.tiles_a ? kt.a_end : kt.end_b;
+    bf16x8 vf[EB];
+#pragma unroll
+    for (int eb = 0; eb < EB; ++eb)
+#pragma unroll
+      for (int u = 0; u < 2; ++u) {
+        bf16x4 quad = bf16x4{(bf16_t)0.f, (bf16_t)0.f, (bf16_t)0.f, (bf16_t)0.f};
+        if (cur.have[u]) quad = *(const bf16x4*)(v_cache + cur.vbase[u] + (size_t)(16 * eb + c) * 4);
+#pragma unroll
+        for (int i = 0; i < 4; ++i) vf[eb][4 * u + i] = quad[i];
+      }
+    if (t + 1 < t_end) load_keys<DC, E>(nxt, kt, t + 1, pages, page_size, n_kv, g, k_cache);
     floatx4 s[2];
-    size_t vbase[2];
-    bool have[2];
 #pragma unroll
     for (int u = 0; u < 2; ++u) {
-      const int ju = j0 + 16 * u;
-      have[u] = ju < end;
       s[u] = floatx4{0.f, 0.f, 0.f, 0.f};
-      vbase[u] = 0;
-      if (have[u]) {
-        const int page = pages[ju / page_size];
-        const size_t head = ((size_t)page * n_kv + g) * page_size;
-        const int off = ju % page_size;
-        const bf16_t* kp = k_cache + (head + off + c) * D + 8 * g4;
 #pragma unroll
-        for (int dc = 0; dc < DC; ++dc)
-          s[u] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(*(const bf16x8*)(kp + 32 * dc), qf[dc], s[u], 0, 0, 0);
-        vbase[u] = head * E + (size_t)((off >> 2) + g4) * E * 4;
-      }
+      for (int dc = 0; dc < DC; ++dc)
+        s[u] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(cur.k[u][dc], qf[dc], s[u], 0, 0, 0);
     }
     float tmax = NEG_INF;
 #pragma unroll
     for (int u = 0; u < 2; ++u)
 #pragma unroll
       for (int i = 0; i < 4; ++i) {
-        const int j = j0 + 16 * u + 4 * g4 + i;
-        const bool ok = have[u] && seen && j < end && sees(pos, j, window, keep_first);
+        const int j = cur.j0 + 16 * u + 4 * g4 + i;
+        const bool ok = cur.have[u] && seen && j < cur.end && sees(pos, j, window, keep_first);
         s[u][i] = ok ? s[u][i] * scale : NEG_INF;
         tmax = fmaxf(tmax, s[u][i]);
       }
@@ -317,18 +358,11 @@ __device__ __forceinline__ void attend_tiles(const KeyTiles& kt, int t_begin, in
     run.m = m_new;
 #pragma unroll
     for (int eb = 0; eb < EB; ++eb) {
-      bf16x8 vf;
-#pragma unroll
-      for (int u = 0; u < 2; ++u) {
-        bf16x4 quad = bf16x4{(bf16_t)0.f, (bf16_t)0.f, (bf16_t)0.f, (bf16_t)0.f};
-        if (have[u]) quad = *(const bf16x4*)(v_cache + vbase[u] + (size_t)(16 * eb + c) * 4);
-#pragma unroll
-        for (int i = 0; i < 4; ++i) vf[4 * u + i] = quad[i];
-      }
 #pragma unroll
       for (int i = 0; i < 4; ++i) run.o[eb][i] *= corr;
-      run.o[eb] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(vf, pf, run.o[eb], 0, 0, 0);
+      run.o[eb] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(vf[eb], pf, run.o[eb], 0, 0, 0);
     }
+    cur = nxt;
   }
 }
 

@@ -69,6 +69,7 @@ class DispatchRules:
     # 2,048 rows, 7 heads of 64 x 128: 1.53 ms in one run.
     scan_min_chunk: int = 16
     scan_max_chunk: int = 64
+    scan_blocks_per_cu: int = 4
     # Windowed attention with a sink: a request that brings at least this many rows to a step is
     # served by the matrix-core kernel (tiles of 16 rows of one request), the others row by row
     # by the plain kernel.  64 decoding requests in tiles of 16 rows of 16 requests: 14.3 ms a

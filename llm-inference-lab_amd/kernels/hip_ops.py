@@ -1162,7 +1162,7 @@ class HipOps:
             return 0
         per_chunk = num_heads * ((value_dim + 63) // 64)
         chunk = self.rules.scan_max_chunk
-        while chunk > self.rules.scan_min_chunk and (rows // chunk) * per_chunk < 4 * self.num_cus:
+        while chunk > self.rules.scan_min_chunk and (rows // chunk) * per_chunk < self.rules.scan_blocks_per_cu * self.num_cus:
             chunk //= 2
         return chunk
 

@@ -102,11 +102,17 @@ class SublayerNormBlock(Block):
             self.ops.add_pending(residual, pending)
             ctx.pending = None
 
-    def _input(self, residual, ctx):
-        """The stream as the sublayers' products read it."""
+    NOTE = "sublayer_norm.copy"      # in the step's notes: the run whose last sum left the stream's copy behind
+
+    def _input(self, residual, ctx, entry):
+        """The stream as the sublayers' products read it: the stream itself in float32, else its
+        rounded copy, which the run just before this one has left behind if it was of this kind."""
         if self.dtype == torch.float32:
             return residual
         h = ctx.scratch("block.stream_copy", tuple(residual.shape), self.dtype)
+        memo = getattr(ctx, "memo", None)
+        if memo is not None and memo.pop(self.NOTE, None) == entry.index - 1:
+            return h
         self.ops.activation(residual, h, "cast")
         return h
 
@@ -122,16 +128,17 @@ class SublayerNormBlock(Block):
 
     def forward(self, residual, ctx, entry):
         self._fold(residual, ctx)
-        h = self._input(residual, ctx)
-        y = self._sublayer(self.mixer, h, residual, ctx, entry)
-        if self.feed_forward is None:
-            self.norm1.add_into(y, residual)
-            return
-        # the sum's new rows go to the feed-forward in the same pass
+        h = self._input(residual, ctx, entry)
+        # every sum's new rows go to the next reader of the stream in the same pass
         copy = h if self.dtype != torch.float32 else None
+        y = self._sublayer(self.mixer, h, residual, ctx, entry)
         self.norm1.add_into(y, residual, copy)
-        y = self._sublayer(self.feed_forward, h, residual, ctx)
-        self.norm2.add_into(y, residual)
+        if self.feed_forward is not None:
+            y = self._sublayer(self.feed_forward, h, residual, ctx)
+            self.norm2.add_into(y, residual, copy)
+        memo = getattr(ctx, "memo", None)
+        if memo is not None and copy is not None:
+            memo[self.NOTE] = entry.index
 
     def weight_bytes(self):
         return sum(p.weight_bytes() for p in self.parts())
