@@ -86,8 +86,8 @@ __device__ __forceinline__ bool find_chunk(const ScanArgs& a, int index, int& fi
   return false;
 }
 
-template <int MODE, bool UNIFORM>
-__global__ __launch_bounds__(1024) void gla_scan_kernel(ScanArgs a) {
+template <int MODE, bool UNIFORM, int THREADS>
+__global__ __launch_bounds__(THREADS) void gla_scan_kernel(ScanArgs a) {
   const int h = blockIdx.y;
   const int e = blockIdx.z * a.cols + (int)(threadIdx.x % a.cols);
   // UNIFORM: a wave lies within one slice (cols a multiple of 64), so the slice's decays,
@@ -110,21 +110,41 @@ __global__ __launch_bounds__(1024) void gla_scan_kernel(ScanArgs a) {
     S[i] = (MODE != SCAN_LOCAL && d0 + i < D) ? st[(size_t)i * E] : 0.f;
     P[i] = 1.f;
   }
+  // A row's decays, keys, queries and value are asked for one row ahead, so that their way
+  // from memory overlaps the sums of the row before.
   const bool whole = d0 + SLICE <= D;
-  for (int t = first; t < last; ++t) {
+  float an[SLICE], kn[SLICE], qn[SLICE], vn = 0.f;
+  auto fetch = [&](int t) {
     const float* row = a.proj + (size_t)t * a.ld;
     const float* qp = row + a.off_q + h * D + d0;
     const float* kp = row + a.off_k + h * D + d0;
     const float* ap = a.decay + ((size_t)t * a.n_heads + h) * D + d0;
-    const float v = row[a.off_v + h * E + e];
+    vn = row[a.off_v + h * E + e];
+#pragma unroll
+    for (int i = 0; i < SLICE; ++i) {
+      const bool in = whole || d0 + i < D;
+      an[i] = in ? ap[i] : 1.f;
+      kn[i] = in ? kp[i] : 0.f;
+      if (MODE != SCAN_LOCAL) qn[i] = in ? qp[i] : 0.f;
+    }
+  };
+  if (first < last) fetch(first);
+  for (int t = first; t < last; ++t) {
+    float ac[SLICE], kc[SLICE], qc[SLICE];
+    const float v = vn;
+#pragma unroll
+    for (int i = 0; i < SLICE; ++i) {
+      ac[i] = an[i];
+      kc[i] = kn[i];
+      if (MODE != SCAN_LOCAL) qc[i] = qn[i];
+    }
+    if (t + 1 < last) fetch(t + 1);
     float acc = 0.f;
 #pragma unroll
     for (int i = 0; i < SLICE; ++i) {
-      if (whole || d0 + i < D) {
-        S[i] = fmaf(ap[i], S[i], kp[i] * v);
-        if (MODE == SCAN_LOCAL) P[i] *= ap[i];
-        else acc = fmaf(S[i], qp[i] * a.q_scale, acc);
-      }
+      S[i] = fmaf(ac[i], S[i], kc[i] * v);
+      if (MODE == SCAN_LOCAL) P[i] *= ac[i];
+      else acc = fmaf(S[i], qc[i] * a.q_scale, acc);
     }
     if (MODE != SCAN_LOCAL) a.parts[(((size_t)t * a.n_heads + h) * a.slices + s) * E + e] = acc;
   }
@@ -187,10 +207,16 @@ extern "C" int llmlab_gla_scan(const float* proj, int ld, int off_q, int off_k, 
   const bool uniform = cols == 64;
   dim3 block(slices * cols);
   const unsigned slabs = (E + cols - 1) / cols;
-#define LLMLAB_SCAN(MODE, GRIDX)                                                                              \
-  do {                                                                                                        \
-    if (uniform) hipLaunchKernelGGL((gla_scan_kernel<MODE, true>), dim3(GRIDX, n_heads, slabs), block, 0, stream, a); \
-    else hipLaunchKernelGGL((gla_scan_kernel<MODE, false>), dim3(GRIDX, n_heads, slabs), block, 0, stream, a);  \
+  // (blocks of up to 256 threads, heads of up to 64 key channels, are compiled with the
+  // registers that leaves them: the rows fetched ahead stay in registers then)
+  const bool small = slices * cols <= 256;
+#define LLMLAB_SCAN(MODE, GRIDX)                                                                                  \
+  do {                                                                                                            \
+    const dim3 grid_(GRIDX, n_heads, slabs);                                                                      \
+    if (uniform && small) hipLaunchKernelGGL((gla_scan_kernel<MODE, true, 256>), grid_, block, 0, stream, a);     \
+    else if (uniform) hipLaunchKernelGGL((gla_scan_kernel<MODE, true, 1024>), grid_, block, 0, stream, a);        \
+    else if (small) hipLaunchKernelGGL((gla_scan_kernel<MODE, false, 256>), grid_, block, 0, stream, a);          \
+    else hipLaunchKernelGGL((gla_scan_kernel<MODE, false, 1024>), grid_, block, 0, stream, a);                    \
   } while (0)
   if (chunk <= 0) {
     LLMLAB_SCAN(SCAN_WHOLE, n_reqs);

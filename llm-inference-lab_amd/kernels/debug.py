@@ -65,11 +65,12 @@ class DispatchRules:
     # The scan of a recurrent mixer (gated linear attention) walks a request's rows one after
     # the other; from twice ``scan_min_chunk`` rows on a request's rows are cut into chunks that
     # run side by side and are joined afterwards (the rows are walked twice then), chunks of at
-    # most ``scan_max_chunk`` rows, shorter while that leaves compute units without blocks.
-    # 2,048 rows, 7 heads of 64 x 128: 1.53 ms in one run.
+    # most ``scan_max_chunk`` rows, shorter while that leaves fewer than ``scan_blocks_per_cu``
+    # blocks to a compute unit.  2,048 rows, 7 heads of 64 x 128: 1.53 ms in one run, 0.17 ms in
+    # chunks of 16 (the pass that joins 128 chunks takes 40 us of it), 0.13 ms in chunks of 64.
     scan_min_chunk: int = 16
     scan_max_chunk: int = 64
-    scan_blocks_per_cu: int = 4
+    scan_blocks_per_cu: int = 1
     # Windowed attention with a sink: a request that brings at least this many rows to a step is
     # served by the matrix-core kernel (tiles of 16 rows of one request), the others row by row
     # by the plain kernel.  64 decoding requests in tiles of 16 rows of 16 requests: 14.3 ms a
