@@ -89,6 +89,7 @@ struct SkinnyArgs {
   // (no residual, bias in group 0) in out[s][M][ldo], part_stride numbers apart.
   int ksplit;
   size_t part_stride;
+  int act;         // SK_STORE only: 1 = max(z, 0)^2 before the rounding
   int tiles;       // tiles of 16 MB rows
   int col_blocks;  // blocks that a tile of rows takes (sets of columns, times ksplit)
 };
@@ -464,7 +465,7 @@ __global__ __launch_bounds__(MB >= 4 ? 512 : 1024) void skinny_block_kernel(Skin
       tile[idx] = sum;
     } else if (nn < a.N) {
       const size_t at = (size_t)m * a.ldo + nn;
-      if (EPI == SK_STORE) ((bf16_t*)a.out)[at] = (bf16_t)sum;
+      if (EPI == SK_STORE) ((bf16_t*)a.out)[at] = (bf16_t)(a.act ? fmaxf(sum, 0.f) * fmaxf(sum, 0.f) : sum);
       else if (EPI == SK_RESID) {
         float old = resid_old;
         if (idx != (int)threadIdx.x) {
@@ -725,6 +726,8 @@ extern "C" int llmlab_skinny_linear(const void* x, int norm, const int* x_rows, 
                                     hipStream_t stream) {
   LLMLAB_REQUIRE(M >= 0 && M <= SK_MAX_ROWS, "skinny_linear: takes at most %d rows, got %d", SK_MAX_ROWS, M);
   LLMLAB_REQUIRE(N > 0 && K > 0 && K % 8 == 0, "skinny_linear: bad sizes N=%d K=%d (K must be a multiple of 8)", N, K);
+  const int act = epilogue == 6 ? 1 : 0;      // (6 at this interface: STORE through the squared relu)
+  if (act) epilogue = SK_STORE;
   LLMLAB_REQUIRE(epilogue >= 0 && epilogue <= 5, "skinny_linear: unknown epilogue %d", epilogue);
   LLMLAB_REQUIRE(pend_splits >= 0 && (pend_splits == 0 || (pend != nullptr && (norm || epilogue == SK_RESID))),
                  "skinny_linear: pending sums go with a norm or into the residual");
@@ -779,6 +782,7 @@ extern "C" int llmlab_skinny_linear(const void* x, int norm, const int* x_rows, 
   a.pend = pend; a.pend_splits = pend_splits; a.pend_ld = pend_ld; a.pend_stride = pend_stride;
   a.ksplit = ksplit; a.part_stride = part_stride; a.tiles = tiles; a.col_blocks = blocks;
   a.qsplit = shape.qsplit;
+  a.act = act;
   a.x = x; a.x_rows = x_rows; a.norm_w = norm_w; a.W = (const bf16_t*)w; a.bias = bias; a.out = out;
   a.inv_freq = inv_freq; a.positions = positions; a.row_req = row_req; a.table = table;
   a.kcache = (bf16_t*)kcache; a.vcache = (bf16_t*)vcache;

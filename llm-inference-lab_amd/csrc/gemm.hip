@@ -70,7 +70,14 @@ struct EpiArgs {
   bf16_t* kcache;
   bf16_t* vcache;
   int table_stride, page_size, nq, nkv, d;
+  // STORE only: 1 = the sum goes through max(z, 0)^2 (in float32) before it is rounded
+  int act;
 };
+
+__device__ __forceinline__ float relu2_f(float z) {
+  z = fmaxf(z, 0.f);
+  return z * z;
+}
 
 __device__ __forceinline__ float silu_f(float z) { return z / (1.f + __expf(-z)); }
 
@@ -80,7 +87,7 @@ __device__ __forceinline__ void epi_store(const EpiArgs& e, int m, int n, float 
   if (e.bias) acc += load_vec(e.bias, e.bias_bf16, n);
   const size_t at = (size_t)m * e.ldo + n;
   if (EPI == EPI_STORE)
-    ((T*)e.out)[at] = from_float<T>(acc);
+    ((T*)e.out)[at] = from_float<T>(e.act ? relu2_f(acc) : acc);
   else if (EPI == EPI_RESID)
     ((float*)e.out)[at] += acc;
   else
@@ -251,6 +258,9 @@ __device__ __forceinline__ void tile_epilogue(const float* Cs, const EpiArgs& e,
       const size_t at = (size_t)m * e.ldo + n;
       const bool whole = vec && n + 4 <= N;
       if constexpr (EPI == EPI_STORE) {
+        if (e.act)
+#pragma unroll
+          for (int q = 0; q < 4; ++q) v[q] = relu2_f(v[q]);
         bf16_t* dst = (bf16_t*)e.out + at;
         if (whole) {
           bf16x4 o;
@@ -1352,6 +1362,9 @@ extern "C" int llmlab_linear(const void* x, const void* w, int dtype, int epilog
                              const void* bias, int bias_dtype, int M, int N, int K, int ldo, int n_out,
                              int num_cus, hipStream_t stream) {
   LLMLAB_REQUIRE(M >= 0 && N > 0 && K > 0, "linear: bad sizes M=%d N=%d K=%d", M, N, K);
+  // 6 at this interface: STORE with the squared-relu activation on the way
+  const int act = epilogue == 6 ? 1 : 0;
+  if (act) epilogue = EPI_STORE;
   LLMLAB_REQUIRE(epilogue >= 0 && epilogue <= 3, "linear: unknown epilogue %d", epilogue);
   if (epilogue == EPI_SWIGLU) {
     LLMLAB_REQUIRE(N % 32 == 0 && n_out > 0 && 2 * ((n_out + 15) / 16 * 16) == N,
@@ -1363,7 +1376,7 @@ extern "C" int llmlab_linear(const void* x, const void* w, int dtype, int epilog
   LLMLAB_REQUIRE(ldo >= n_out, "linear: output row stride %d < %d columns", ldo, n_out);
   if (M == 0) return 0;
   EpiArgs e{out, bias, bias_dtype == DT_BF16, ldo, n_out, 0, 0,
-            nullptr, nullptr, nullptr, nullptr, nullptr, nullptr, 0, 0, 0, 0, 0};
+            nullptr, nullptr, nullptr, nullptr, nullptr, nullptr, 0, 0, 0, 0, 0, act};
   if (num_cus <= 0) num_cus = 256;
   if (dtype == DT_BF16) {
     LLMLAB_REQUIRE(K % 8 == 0, "linear(bfloat16): inner size %d must be a multiple of 8", K);

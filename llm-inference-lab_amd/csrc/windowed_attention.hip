@@ -243,8 +243,8 @@ struct Running {
 // prefix [0, a_end), then [b_start, p_hi] (p_lo, p_hi: the lowest and highest position among
 // the queries; b_start: the lowest window's first key rounded down to 16).
 struct KeyTiles {
-  int a_end, b_start, end_b, tiles_a, tiles;
-  __device__ KeyTiles(int p_lo, int p_hi, int window, int keep_first) {
+  int a_end, b_start, end_b, tiles_a, tiles, p_lo, p_hi;
+  __device__ KeyTiles(int p_lo_, int p_hi_, int window, int keep_first) : p_lo(p_lo_), p_hi(p_hi_) {
     const int lo = window > 0 ? (p_lo - window + 1 > 0 ? p_lo - window + 1 : 0) : 0;
     b_start = lo & ~15;
     a_end = keep_first < b_start ? keep_first : b_start;
@@ -328,15 +328,29 @@ __device__ __forceinline__ void attend_tiles(const KeyTiles& kt, int t_begin, in
         s[u] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(cur.k[u][dc], qf[dc], s[u], 0, 0, 0);
     }
     float tmax = NEG_INF;
+    // a whole tile that every query of the wave sees (behind the lowest position, inside the
+    // window of the highest or the kept prefix) needs no mask key by key: most tiles of a long window
+    const bool interior = cur.have[1] && cur.j0 + 31 < cur.end && cur.j0 + 31 <= kt.p_lo &&
+                          (window <= 0 || kt.p_hi - cur.j0 < window || cur.j0 + 31 < keep_first);
+    if (interior) {
 #pragma unroll
-    for (int u = 0; u < 2; ++u)
+      for (int u = 0; u < 2; ++u)
 #pragma unroll
-      for (int i = 0; i < 4; ++i) {
-        const int j = cur.j0 + 16 * u + 4 * g4 + i;
-        const bool ok = cur.have[u] && seen && j < cur.end && sees(pos, j, window, keep_first);
-        s[u][i] = ok ? s[u][i] * scale : NEG_INF;
-        tmax = fmaxf(tmax, s[u][i]);
-      }
+        for (int i = 0; i < 4; ++i) {
+          s[u][i] = seen ? s[u][i] * scale : NEG_INF;
+          tmax = fmaxf(tmax, s[u][i]);
+        }
+    } else {
+#pragma unroll
+      for (int u = 0; u < 2; ++u)
+#pragma unroll
+        for (int i = 0; i < 4; ++i) {
+          const int j = cur.j0 + 16 * u + 4 * g4 + i;
+          const bool ok = cur.have[u] && seen && j < cur.end && sees(pos, j, window, keep_first);
+          s[u][i] = ok ? s[u][i] * scale : NEG_INF;
+          tmax = fmaxf(tmax, s[u][i]);
+        }
+    }
     tmax = fmaxf(tmax, __shfl_xor(tmax, 16, WAVE));
     tmax = fmaxf(tmax, __shfl_xor(tmax, 32, WAVE));
     const float m_new = fmaxf(run.m, tmax);

@@ -22,6 +22,7 @@ from .debug import DispatchRules, KernelDebug
 
 DT_F32, DT_BF16 = 0, 1
 EPI_STORE, EPI_RESID, EPI_F32, EPI_SWIGLU, EPI_QKV, EPI_PART = 0, 1, 2, 3, 4, 5
+EPI_RELU2 = 6        # STORE through max(z, 0)^2, taken on the float32 sum
 
 _c_int, _c_long, _c_float, _c_size, _c_ptr = (ctypes.c_int, ctypes.c_long, ctypes.c_float,
                                               ctypes.c_size_t, ctypes.c_void_p)
@@ -462,7 +463,7 @@ class HipOps:
         if x.dtype == torch.bfloat16 and k % 8 != 0:
             raise UnsupportedSizeError(
                 f"bfloat16 matrix products need an inner size that is a multiple of 8, got {k}")
-        want_out = x.dtype if epilogue in (EPI_STORE, EPI_SWIGLU) else torch.float32
+        want_out = x.dtype if epilogue in (EPI_STORE, EPI_SWIGLU, EPI_RELU2) else torch.float32
         if out.dtype != want_out:
             raise TypeError(f"linear: output must be {want_out}, got {out.dtype}")
         if bias is not None:
@@ -484,6 +485,11 @@ class HipOps:
 
     def linear(self, x, w, out, bias=None) -> None:
         self._linear(x, w, out, bias, EPI_STORE, w.shape[0])
+
+    def linear_relu2(self, x, w, out) -> None:
+        """``out = max(x w^T, 0) ** 2`` in the compute dtype: the activation is taken on the float32
+        sums and rounded once."""
+        self._linear(x, w, out, None, EPI_RELU2, w.shape[0])
 
     def linear_residual(self, x, w, resid, bias=None, pending: Optional[PendingSums] = None) -> None:
         """``resid += x w^T (+ bias)``, and the pending pieces of ``resid`` with it."""

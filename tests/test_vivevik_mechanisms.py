@@ -69,6 +69,20 @@ def test_squared_relu(backend, dtype):
     close(out, x.cpu().to(F64), dtype, "cast")
 
 
+@pytest.mark.parametrize("backend", BACKENDS)
+@pytest.mark.parametrize("dtype", DTYPES)
+@pytest.mark.parametrize("rows", [1, 9, 40, 300])
+def test_squared_relu_as_the_epilogue_of_a_product(backend, dtype, rows):
+    """Few rows and many (the product kernels differ), both dtypes: the activation is taken on
+    the float32 sums."""
+    ops = ops_of(backend)
+    x = randn(rows, 72, seed=5).to(dtype)
+    w = randn(200, 72, seed=6, scale=0.3).to(dtype)
+    out = torch.empty(rows, 200, dtype=dtype, device=ops.device)
+    ops.linear_relu2(x.to(ops.device), ops.prepare_weight(w.to(ops.device)), out)
+    close(out, P.squared_relu_mlp(x.to(F64), w.to(F64), torch.eye(200, dtype=F64)), dtype, "relu(x W^T)^2", f32=2e-5)
+
+
 # ------------------------------------------------------------------ attention
 class Paged:
     """Keys and values of a few requests in pages handed out in a scattered order."""
