@@ -111,42 +111,45 @@ __global__ __launch_bounds__(THREADS) void gla_scan_kernel(ScanArgs a) {
     P[i] = 1.f;
   }
   // A row's decays, keys, queries and value are asked for one row ahead, so that their way
-  // from memory overlaps the sums of the row before.
+  // from memory overlaps the sums of the row before; two sets of registers take turns, so
+  // nothing is copied.
   const bool whole = d0 + SLICE <= D;
-  float an[SLICE], kn[SLICE], qn[SLICE], vn = 0.f;
-  auto fetch = [&](int t) {
+  struct Row {
+    float a[SLICE], k[SLICE], q[SLICE], v;
+  };
+  auto fetch = [&](Row& r, int t) {
     const float* row = a.proj + (size_t)t * a.ld;
     const float* qp = row + a.off_q + h * D + d0;
     const float* kp = row + a.off_k + h * D + d0;
     const float* ap = a.decay + ((size_t)t * a.n_heads + h) * D + d0;
-    vn = row[a.off_v + h * E + e];
+    r.v = row[a.off_v + h * E + e];
 #pragma unroll
     for (int i = 0; i < SLICE; ++i) {
       const bool in = whole || d0 + i < D;
-      an[i] = in ? ap[i] : 1.f;
-      kn[i] = in ? kp[i] : 0.f;
-      if (MODE != SCAN_LOCAL) qn[i] = in ? qp[i] : 0.f;
+      r.a[i] = in ? ap[i] : 1.f;
+      r.k[i] = in ? kp[i] : 0.f;
+      if (MODE != SCAN_LOCAL) r.q[i] = in ? qp[i] : 0.f;
     }
   };
-  if (first < last) fetch(first);
-  for (int t = first; t < last; ++t) {
-    float ac[SLICE], kc[SLICE], qc[SLICE];
-    const float v = vn;
-#pragma unroll
-    for (int i = 0; i < SLICE; ++i) {
-      ac[i] = an[i];
-      kc[i] = kn[i];
-      if (MODE != SCAN_LOCAL) qc[i] = qn[i];
-    }
-    if (t + 1 < last) fetch(t + 1);
+  auto take = [&](const Row& r, int t) {
     float acc = 0.f;
 #pragma unroll
     for (int i = 0; i < SLICE; ++i) {
-      S[i] = fmaf(ac[i], S[i], kc[i] * v);
-      if (MODE == SCAN_LOCAL) P[i] *= ac[i];
-      else acc = fmaf(S[i], qc[i] * a.q_scale, acc);
+      S[i] = fmaf(r.a[i], S[i], r.k[i] * r.v);
+      if (MODE == SCAN_LOCAL) P[i] *= r.a[i];
+      else acc = fmaf(S[i], r.q[i], acc);
     }
-    if (MODE != SCAN_LOCAL) a.parts[(((size_t)t * a.n_heads + h) * a.slices + s) * E + e] = acc;
+    if (MODE != SCAN_LOCAL) a.parts[(((size_t)t * a.n_heads + h) * a.slices + s) * E + e] = acc * a.q_scale;
+  };
+  Row r0, r1;
+  if (first < last) fetch(r0, first);
+  for (int t = first; t < last; t += 2) {
+    if (t + 1 < last) fetch(r1, t + 1);
+    take(r0, t);
+    if (t + 1 < last) {
+      if (t + 2 < last) fetch(r0, t + 2);
+      take(r1, t + 1);
+    }
   }
   if (MODE == SCAN_FINISH) return;
 #pragma unroll
