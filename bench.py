@@ -147,15 +147,17 @@ def vivevik_flops(cfg, tokens):
     return total + 2 * w * cfg.vocab
 
 
-def design_run(args):
-    """``--design vivevik``: both models at each size, one after the other on the same GPU."""
+def design_run(args, bracket=None):
+    """``--design vivevik``: both models at each size, one after the other on the same GPU.
+    ``--only-model``, ``--only-prefill`` / ``--only-decode`` and ``--batch`` narrow the run (for
+    profiles: ``--profile`` collects the timed steps only)."""
     import types
     import torch
     import llm_inference_lab_amd as lab
     from llm_inference_lab_amd.config import get_architecture
     from llm_inference_lab_amd.engine.model import CausalLM
     context = args.context or 2048
-    batches = sorted({8, 64})
+    batches = [args.batch] if args.only_decode else sorted({8, 64})
     record = {}
     for size in ([args.size] if args.size else list(DESIGN_SIZES)):
         width, heads, kv, dim, ff, layers = DESIGN_SIZES[size]
@@ -165,6 +167,8 @@ def design_run(args):
         record[size] = {"width": width, "heads": heads, "kv_heads": kv, "head_dim": dim, "ff": ff, "layers": layers,
                         "context": context, "window": DESIGN_WINDOW}
         for label, cfg in (("vivevik", vivevik_config(size)), ("qwen2", qwen)):
+            if args.only_model and label != args.only_model:
+                continue
             expected = CausalLM(get_architecture(cfg.architecture).build_spec(cfg)).tensor_specs()
             arch = get_architecture(cfg.architecture)
             drawn = (arch.random_init(cfg, expected, 0, torch.bfloat16) if arch.random_init is not None
@@ -174,15 +178,16 @@ def design_run(args):
                                 max_batch_tokens=FILL_TOKENS, max_seq_len=context + PAGE,
                                 graph=False if args.no_graph else args.graph)
             view = types.SimpleNamespace(vocab_size=engine.spec.vocab_size)
-            runs = Runs(engine, view, context, args.dtype, args.samples)
+            runs = Runs(engine, view, context, args.dtype, args.samples, bracket)
             flops = vivevik_flops(cfg, args.prefill_tokens) if label == "vivevik" else prefill_flops(cfg, args.prefill_tokens)
-            out = {"prefill": runs.prefill(args.prefill_tokens, flops=flops),
-                   "weight_bytes_per_step": engine.weight_bytes_per_step()}
+            out = {"weight_bytes_per_step": engine.weight_bytes_per_step()}
+            if not args.only_decode:
+                out["prefill"] = runs.prefill(args.prefill_tokens, flops=flops)
             # what a decode step has to move: the weights once, of every request the cache its
             # layers still see (a windowed group: the window and the kept prefix) and its
             # recurrent states, read and written
             state = 2 * sum(t[0].numel() * t.element_size() for per in engine.cache.state.values() for t in per.values())
-            for b in batches:
+            for b in ([] if args.only_prefill else batches):
                 seconds, live, ms = runs.decode_samples(b, args.steps, args.warmup)
                 seen = sum(len(g.entries) * g.spec.bytes_per_token(engine.cache.dtype)
                            * min(live / b, (g.window + g.spec.keep_first) if g.window else live / b)
@@ -708,6 +713,8 @@ def main():
     ap.add_argument("--design", choices=["vivevik"], default=None,
                     help="throughput of another design beside the Qwen2 decoder of equal size")
     ap.add_argument("--size", choices=sorted(DESIGN_SIZES), default=None, help="--design: one size only")
+    ap.add_argument("--only-model", choices=["vivevik", "qwen2"], default=None, help="--design: one of the two models only")
+    ap.add_argument("--only-decode", action="store_true", help="--design: decode at --batch only, no prefill")
     ap.add_argument("--side", choices=["7b", "32b", "f32", "peaks"], help=argparse.SUPPRESS)
     args = ap.parse_args()
     if args.gpus != 1:
@@ -720,7 +727,7 @@ def main():
         side_run(args)
         return
     if args.design:
-        design_run(args)
+        design_run(args, bracket)
         return
 
     # The other shapes and the other dtype are points of the default line: each runs as a
