@@ -140,6 +140,33 @@ def test_greedy_generation_through_the_scheduler(backend, name):
     assert m["rows_used"] == 0 and all(g["pages_used"] == 0 for g in m["groups"])
 
 
+@pytest.mark.gpu
+@pytest.mark.parametrize("dtype", ["f32", "bf16"])
+def test_decode_steps_replayed_from_a_graph(dtype):
+    """Decode steps captured into a HIP graph and replayed, with the program's own eager steps
+    (new requests' prompts) between the replays: every token the one an engine without graphs
+    generates, and in float32 the plain implementation's."""
+    name = "P"
+    cfg = V.config_of(name)
+    tensors = V.make_tensors(cfg, 1)
+    prompts = [V.random_ids(cfg, n, 70 + n) for n in (5, 21, 40, 9)]
+    runs = {}
+    for graph in (False, True):
+        engine = V.make_engine(name, 1, dtype, page_size=16, num_pages=40, max_requests=2, max_batch_tokens=32, graph=graph)
+        runs[graph] = engine.generate(prompts, max_new_tokens=40)
+        if graph:
+            assert engine.metrics()["graphs"]["replays"] > 20
+    assert runs[True] == runs[False]
+    if dtype == "f32":
+        for prompt, tokens in zip(prompts[:2], runs[True]):
+            ids = list(prompt)
+            for n, token in enumerate(tokens):
+                logits = plain_vivevik.forward(ids, tensors, cfg.to_dict())[-1]
+                best = int(logits.argmax())
+                assert token == best or float(logits[best] - logits[token]) < 2 * TOL["f32"], (n, token, best)
+                ids.append(token)
+
+
 def test_configuration_round_trip_and_errors():
     for name, raw in V.CONFIGS.items():
         cfg = V.config_of(name)
