@@ -103,11 +103,11 @@ def prefill_flops(cfg, tokens):
 # Layer sizes for ``--design vivevik``: (width, heads, kv heads, head size, feed-forward width,
 # layers).  Layers come in threes: a recurrent layer without a feed-forward, an attention layer
 # with keys and values of its own, and one that reads the former's; windows of 1,024 positions
-# that keep the first four.
+# that keep the first eight.
 DESIGN_SIZES = {"small": (896, 14, 2, 64, 4864, 12), "medium": (2048, 16, 2, 128, 11008, 12),
                 "large": (3584, 28, 4, 128, 18944, 6)}
 DESIGN_VOCAB = 32000
-DESIGN_WINDOW, DESIGN_KEEP = 1024, 4
+DESIGN_WINDOW, DESIGN_KEEP = 1024, 8
 
 
 def vivevik_config(size):
@@ -117,7 +117,7 @@ def vivevik_config(size):
     for i in range(layers):
         if i % 3 == 0:
             listed.append(dict(type="gla", mlp=None,
-                               mixer=dict(heads=width // 128, dim=64, vdim=128, tau=16.0, rank=16)))
+                               mixer=dict(heads=width // 128, dim=64, vdim=128, tau=8.0, rank=32)))
         else:
             mixer = dict(heads=heads, kv_heads=kv, dim=dim, vdim=dim, scale=dim ** -0.5,
                          mask=dict(size=DESIGN_WINDOW, keep_first=DESIGN_KEEP))
@@ -135,7 +135,7 @@ def vivevik_flops(cfg, tokens):
     for l in cfg.layers:
         if l.type == "gla":
             qk, v = l.heads * l.dim, l.heads * l.vdim
-            total += tokens * 2 * (w * (2 * qk + 2 * v + (l.rank or 16)) + v * w + (l.rank or 16) * qk)
+            total += tokens * 2 * (w * (2 * qk + 2 * v + (l.rank or 32)) + v * w + (l.rank or 32) * qk)
             total += tokens * 4 * l.heads * l.dim * l.vdim
         else:
             q, k, v = l.heads * l.dim, l.kv_heads * l.dim, l.kv_heads * l.vdim

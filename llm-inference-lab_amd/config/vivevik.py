@@ -53,7 +53,7 @@ class VivevikConfig:
 
     ARCHITECTURE = "Vivevik"
     MAX_POSITIONS = 1 << 20          # the design has no position table: the engine's own bound
-    DEFAULT_DECAY_RANK = 16          # random-weights mode, when the configuration names no rank
+    DEFAULT_DECAY_RANK = 32          # random-weights mode, when the configuration names no rank
 
     @classmethod
     def from_dict(cls, raw: Dict[str, Any], where: str = "config.json") -> "VivevikConfig":
