@@ -1,6 +1,6 @@
 // Attention over a paged cache with a sliding window, a prefix of first positions that
 // stays visible, and a softmax whose denominator holds one more, learned term per head
-// (a "sink": it has no key and no value).  Keys and values may differ in width.  gfx950.
+// (a "sink": a logit that only enlarges the denominator).  Keys and values may differ in width.  gfx950.
 //
 // Pages: keys [page, kv head, P, D] row by row; values [page, kv head, P, E] with the P * E
 // numbers of a (page, kv head) in the order [P / 4][E][4]: the four keys of a quad side by
@@ -89,10 +89,10 @@ extern "C" int llmlab_project_norm_write(const float* proj, int ld, int rows, in
 }
 
 // ------------------------------------------------------------------ attention
-// The query at position i of its request sees key j if j <= i and (i - j < window or
-// j < keep_first); window <= 0: every j <= i.  Scores, the running maximum, the denominator
+// The query at position i of its request attends to the keys i - window < j <= i and to the
+// kept prefix j < min(keep_first, i + 1); window <= 0: every j <= i.  Scores, the running maximum, the denominator
 // and the weighted sum of values are float32.  With a sink the running maximum starts at
-// sink[h] and the denominator at 1 = exp(sink - sink): the term counts once and brings no value.
+// sink[h] and the denominator at 1 = exp(sink - sink), and nothing is added to the weighted sum.
 //
 // Both kernels walk the keys in two runs, each from an aligned start, and mask key by key:
 // the kept prefix [0, min(keep_first, B)) and [B, i], where B is the window's first key

@@ -225,10 +225,12 @@ class WindowedSinkAttention(Mixer):
     (``kv_heads x value_dim``), no biases.  ``qk_norm="whole"``: q, and k alike, is divided by
     the root mean square over its WHOLE width (all heads at once, ``eps`` inside the root)
     and multiplied by a weight of that width, in float32, before it is cut into heads.  The
-    query at position i sees key j if ``j <= i and (i - j < window or j < keep_first)``
+    query at position i attends to the keys ``i - window < j <= i`` and, beside them, to the
+    keys ``j < min(keep_first, i + 1)``
     (``window`` None: every ``j <= i``).  Scores ``q.k * scale``; weights ``exp(s_j - m) /
     (sum_j exp(s_j - m) + exp(sink_h - m))`` where ``sink_h`` is one learned number per head
-    (``sink=False``: the plain softmax): the extra term has no key and no value.  Head ``h``
+    (``sink=False``: the plain softmax): the extra term only enlarges the denominator, nothing is
+    summed for it.  Head ``h``
     reads kv head ``h // (heads / kv_heads)``.  No position encoding enters the scores.
 
     ``own_kv=False``: the layer has no key and value projections; its run reads the pages
