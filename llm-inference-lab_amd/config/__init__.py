@@ -1,13 +1,14 @@
 from .errors import ConfigError, WeightError, UnsupportedSizeError
-from .spec import PartSpec, BlockSpec, ScheduleEntry, ModelSpec
+from .spec import PartSpec, BlockSpec, ScheduleEntry, StreamOffset, ModelSpec
 from .registry import (register_architecture, unregister_architecture, get_architecture,
                        registered_architectures, architecture_of, read_config, Architecture)
 from .qwen2 import Qwen2Config
 from .vivevik import VivevikConfig
+from .ruvalorn import RuvalornConfig
 
 __all__ = [
     "ConfigError", "WeightError", "UnsupportedSizeError", "PartSpec", "BlockSpec",
-    "ScheduleEntry", "ModelSpec", "register_architecture", "unregister_architecture",
+    "ScheduleEntry", "StreamOffset", "ModelSpec", "register_architecture", "unregister_architecture",
     "get_architecture", "registered_architectures", "architecture_of", "read_config",
-    "Architecture", "Qwen2Config", "VivevikConfig",
+    "Architecture", "Qwen2Config", "VivevikConfig", "RuvalornConfig",
 ]

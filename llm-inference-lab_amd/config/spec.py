@@ -39,13 +39,27 @@ class BlockSpec:
 
 
 @dataclasses.dataclass(frozen=True)
+class StreamOffset:
+    """A learned vector that is added to every row of the residual stream: row ``row`` of the
+    tensor ``tensor`` of the model file, a table ``[rows, hidden]``."""
+
+    tensor: str
+    row: int
+    rows: int
+
+
+@dataclasses.dataclass(frozen=True)
 class ScheduleEntry:
     """One run of a block.  ``block`` indexes ``ModelSpec.blocks`` (the same
-    block may run more than once).  ``cache_of`` names an earlier schedule
-    entry whose cache this run reads instead of keeping one of its own."""
+    block may run more than once; every run keeps a cache and a state of its own).
+    ``cache_of`` names an earlier schedule
+    entry whose cache this run reads instead of keeping one of its own.  ``offset``: a vector
+    added to the stream right before this run (a model that runs some of its layers several
+    times tells the passes apart by it)."""
 
     block: int
     cache_of: Optional[int] = None
+    offset: Optional[StreamOffset] = None
 
 
 @dataclasses.dataclass(frozen=True)
@@ -71,3 +85,6 @@ class ModelSpec:
                     raise ValueError(f"schedule[{i}].cache_of must name an earlier entry")
                 if self.schedule[entry.cache_of].cache_of is not None:
                     raise ValueError(f"schedule[{i}].cache_of names an entry that owns no cache")
+            if entry.offset is not None and not 0 <= entry.offset.row < entry.offset.rows:
+                raise ValueError(f"schedule[{i}].offset names row {entry.offset.row} of a table of "
+                                 f"{entry.offset.rows} rows")

@@ -4,7 +4,7 @@
 
 extern "C" const char* llmlab_last_error() { return g_llmlab_error; }
 
-extern "C" int llmlab_abi_version() { return 7; }
+extern "C" int llmlab_abi_version() { return 8; }
 
 // --------------------------------------------------------------- embedding
 // out[r, :] = float(table[ids[r], :]); an id outside [0, vocab) is clamped (the
@@ -583,5 +583,49 @@ extern "C" int llmlab_activation(const float* x, void* out, int out_dtype, int a
   }
 #undef LLMLAB_ACT
   LLMLAB_LAUNCH_CHECK("activation");
+  return 0;
+}
+
+// ------------------------------------------------- one gate per head on a mixer's output
+// out[r, h, :] *= sigmoid(gate[r, h]): the sigmoid and the product in float32, one rounding.
+template <typename T>
+__global__ void gate_heads_kernel(T* __restrict__ out, const float* __restrict__ gate, int heads, int head_dim,
+                                  size_t n) {
+  for (size_t i = (size_t)blockIdx.x * blockDim.x + threadIdx.x; i < n; i += (size_t)gridDim.x * blockDim.x) {
+    const float g = gate[i / head_dim];          // (rows of heads * head_dim numbers, gates [rows, heads])
+    out[i] = from_float<T>(to_float(out[i]) / (1.f + __expf(-g)));
+  }
+}
+
+extern "C" int llmlab_gate_heads(void* out, int dtype, const float* gate, int rows, int heads, int head_dim,
+                                 hipStream_t stream) {
+  LLMLAB_REQUIRE(rows >= 0 && heads > 0 && head_dim > 0, "gate_heads: bad sizes rows=%d heads=%d head_dim=%d", rows,
+                 heads, head_dim);
+  const size_t n = (size_t)rows * heads * head_dim;
+  if (n == 0) return 0;
+  const int blocks = (int)((n + 255) / 256 < 65535 ? (n + 255) / 256 : 65535);
+  if (dtype == DT_BF16)
+    hipLaunchKernelGGL(gate_heads_kernel<bf16_t>, dim3(blocks), dim3(256), 0, stream, (bf16_t*)out, gate, heads,
+                       head_dim, n);
+  else
+    hipLaunchKernelGGL(gate_heads_kernel<float>, dim3(blocks), dim3(256), 0, stream, (float*)out, gate, heads,
+                       head_dim, n);
+  LLMLAB_LAUNCH_CHECK("gate_heads");
+  return 0;
+}
+
+// ------------------------------------------------- one vector added to every row of the stream
+__global__ void add_row_vector_kernel(float* __restrict__ x, const float* __restrict__ v, int hidden, size_t n) {
+  for (size_t i = (size_t)blockIdx.x * blockDim.x + threadIdx.x; i < n; i += (size_t)gridDim.x * blockDim.x)
+    x[i] += v[i % hidden];
+}
+
+extern "C" int llmlab_add_row_vector(float* x, const float* v, int rows, int hidden, hipStream_t stream) {
+  LLMLAB_REQUIRE(rows >= 0 && hidden > 0, "add_row_vector: bad sizes rows=%d hidden=%d", rows, hidden);
+  const size_t n = (size_t)rows * hidden;
+  if (n == 0) return 0;
+  const int blocks = (int)((n + 255) / 256 < 65535 ? (n + 255) / 256 : 65535);
+  hipLaunchKernelGGL(add_row_vector_kernel, dim3(blocks), dim3(256), 0, stream, x, v, hidden, n);
+  LLMLAB_LAUNCH_CHECK("add_row_vector");
   return 0;
 }

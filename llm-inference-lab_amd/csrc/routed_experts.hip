@@ -1,0 +1,134 @@
+// A feed-forward made of many small ones (experts) of which every row uses a few: the choice,
+// the sorting of rows by expert, and the sum of the chosen experts' results, for gfx950.
+//
+//   select      per row: softmax over the router's outputs, choice value = score + correction,
+//               the best groups of neighbours, the top outputs among them; weight = score * scale
+//   add_chosen  resid[r] += (sum of the weights of row r's choices within [first, last)) * src[r]
+#include "common.h"
+
+extern "C" const char* llmlab_last_error() { return g_llmlab_error; }
+
+constexpr int SELECT_MAX_OUTPUTS = 1024;     // router outputs a row's wave keeps in LDS
+
+// One wave a row.  Everything in float32; ties go to the smaller index, as a scan in order does.
+__global__ __launch_bounds__(64) void moe_select_kernel(const float* __restrict__ logits, const float* __restrict__ correction,
+                                                        int outputs, int groups, int keep, int top, float scale,
+                                                        int* __restrict__ chosen, float* __restrict__ weights) {
+  __shared__ float s_score[SELECT_MAX_OUTPUTS], s_choice[SELECT_MAX_OUTPUTS];
+  __shared__ float s_group[SELECT_MAX_OUTPUTS];
+  const int row = blockIdx.x, lane = threadIdx.x;
+  const float* z = logits + (size_t)row * outputs;
+  float m = -INFINITY;
+  for (int e = lane; e < outputs; e += WAVE) m = fmaxf(m, z[e]);
+  for (int o = 32; o > 0; o >>= 1) m = fmaxf(m, __shfl_xor(m, o));
+  float sum = 0.f;
+  for (int e = lane; e < outputs; e += WAVE) {
+    const float p = expf(z[e] - m);
+    s_score[e] = p;
+    sum += p;
+  }
+  for (int o = 32; o > 0; o >>= 1) sum += __shfl_xor(sum, o);
+  const float inv = 1.f / sum;
+  for (int e = lane; e < outputs; e += WAVE) {
+    const float s = s_score[e] * inv;
+    s_score[e] = s;
+    s_choice[e] = s + correction[e];
+  }
+  __syncthreads();
+  const int per = outputs / groups;
+  if (keep < groups) {
+    for (int g = lane; g < groups; g += WAVE) {
+      float best = -INFINITY;
+      for (int i = 0; i < per; ++i) best = fmaxf(best, s_choice[g * per + i]);
+      s_group[g] = best;
+    }
+    __syncthreads();
+    // a group is kept if fewer than `keep` groups come before it in the order (value down, index up)
+    for (int g = lane; g < groups; g += WAVE) {
+      const float mine = s_group[g];
+      int before = 0;
+      for (int o = 0; o < groups; ++o) {
+        const float other = s_group[o];
+        before += (other > mine) || (other == mine && o < g);
+      }
+      if (before >= keep)
+        for (int i = 0; i < per; ++i) s_choice[g * per + i] = -INFINITY;
+    }
+    __syncthreads();
+  }
+  for (int k = 0; k < top; ++k) {
+    float best = -INFINITY;
+    int at = outputs;             // (when every value left is minus infinity: the smallest index left)
+    for (int e = lane; e < outputs; e += WAVE) {
+      const float c = s_choice[e];
+      if (c > best || (c == best && e < at)) {
+        best = c;
+        at = e;
+      }
+    }
+    for (int o = 32; o > 0; o >>= 1) {
+      const float ob = __shfl_xor(best, o);
+      const int oa = __shfl_xor(at, o);
+      if (ob > best || (ob == best && oa < at)) {
+        best = ob;
+        at = oa;
+      }
+    }
+    at = min(at, outputs - 1);
+    if (lane == 0) {
+      chosen[(size_t)row * top + k] = at;
+      weights[(size_t)row * top + k] = s_score[at] * scale;
+      s_choice[at] = -INFINITY;          // taken
+    }
+    __syncthreads();
+  }
+}
+
+extern "C" int llmlab_moe_select(const float* logits, const float* correction, int rows, int outputs, int groups,
+                                 int keep, int top, float scale, int* chosen, float* weights, hipStream_t stream) {
+  LLMLAB_REQUIRE(rows >= 0 && outputs > 0 && outputs <= SELECT_MAX_OUTPUTS,
+                 "moe_select: a router of 1 to %d outputs, got %d", SELECT_MAX_OUTPUTS, outputs);
+  LLMLAB_REQUIRE(groups > 0 && outputs % groups == 0 && keep > 0 && keep <= groups && top > 0 &&
+                     top <= keep * (outputs / groups),
+                 "moe_select: %d outputs in %d groups of which %d are kept, top %d", outputs, groups, keep, top);
+  if (rows == 0) return 0;
+  hipLaunchKernelGGL(moe_select_kernel, dim3(rows), dim3(64), 0, stream, logits, correction, outputs, groups, keep,
+                     top, scale, chosen, weights);
+  LLMLAB_LAUNCH_CHECK("moe_select");
+  return 0;
+}
+
+// resid[r, :] += w_r * src[r, :],  w_r = sum of weights[r, k] over the k with first <= chosen[r, k] < last
+template <typename T>
+__global__ void moe_add_chosen_kernel(float* __restrict__ resid, const T* __restrict__ src, const int* __restrict__ chosen,
+                                      const float* __restrict__ weights, int top, int first, int last, int hidden) {
+  const int row = blockIdx.x;
+  float w = 0.f;
+  bool any = false;
+  for (int k = 0; k < top; ++k) {
+    const int e = chosen[(size_t)row * top + k];
+    if (e >= first && e < last) {
+      w += weights[(size_t)row * top + k];
+      any = true;
+    }
+  }
+  if (!any) return;
+  for (int i = threadIdx.x; i < hidden; i += blockDim.x)
+    resid[(size_t)row * hidden + i] += w * to_float(src[(size_t)row * hidden + i]);
+}
+
+extern "C" int llmlab_moe_add_chosen(float* resid, const void* src, int src_dtype, const int* chosen,
+                                     const float* weights, int rows, int top, int first, int last, int hidden,
+                                     hipStream_t stream) {
+  LLMLAB_REQUIRE(rows >= 0 && top > 0 && hidden > 0, "moe_add_chosen: bad sizes rows=%d top=%d hidden=%d", rows, top,
+                 hidden);
+  if (rows == 0 || first >= last) return 0;
+  if (src_dtype == DT_BF16)
+    hipLaunchKernelGGL(moe_add_chosen_kernel<bf16_t>, dim3(rows), dim3(256), 0, stream, resid, (const bf16_t*)src,
+                       chosen, weights, top, first, last, hidden);
+  else
+    hipLaunchKernelGGL(moe_add_chosen_kernel<float>, dim3(rows), dim3(256), 0, stream, resid, (const float*)src, chosen,
+                       weights, top, first, last, hidden);
+  LLMLAB_LAUNCH_CHECK("moe_add_chosen");
+  return 0;
+}

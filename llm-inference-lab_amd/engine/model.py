@@ -19,7 +19,7 @@ from ..cache.manager import CacheManager, GroupLayout
 from ..config.spec import ModelSpec
 from ..parts.base import NormedInput
 from ..parts.registry import build_part, part_class
-from ..weights.loader import TensorSpec
+from ..weights.loader import TensorSpec, VECTOR
 
 
 @dataclasses.dataclass
@@ -60,6 +60,8 @@ class CausalLM:
         self.final_norm = build_part("norm", spec.final_norm)
         self.head = build_part("head", spec.head)
         self.entries: List[EntryView] = [EntryView(i, e.block) for i, e in enumerate(spec.schedule)]
+        # vectors added to the stream before a run (``ScheduleEntry.offset``): run -> (table, row)
+        self.offsets: Dict[int, Tuple[torch.Tensor, int]] = {}
         self.ops = None
         self.dtype = None
         self._weight_bytes = None          # worked out when first asked for, after the weights are bound
@@ -107,6 +109,9 @@ class CausalLM:
             add(b.tensor_specs())
         add(self.final_norm.tensor_specs())
         add(self.head.tensor_specs())
+        for entry in self.spec.schedule:
+            if entry.offset is not None:
+                add({entry.offset.tensor: TensorSpec((entry.offset.rows, self.spec.hidden_size), VECTOR)})
         return specs
 
     def bind(self, tensors: Dict[str, torch.Tensor], ops, dtype: torch.dtype) -> None:
@@ -117,6 +122,13 @@ class CausalLM:
             b.bind(tensors, ops, dtype)
         self.final_norm.bind(tensors, ops, dtype)
         self.head.bind(tensors, ops, dtype)
+        tables: Dict[str, torch.Tensor] = {}
+        for i, entry in enumerate(self.spec.schedule):
+            if entry.offset is not None:
+                name = entry.offset.tensor
+                if name not in tables:      # (the stream is float32 in both modes, so its offsets are too)
+                    tables[name] = tensors[name].float().contiguous()
+                self.offsets[i] = (tables[name], entry.offset.row)
         ops.release_shared()
 
     def weight_bytes_per_step(self) -> int:
@@ -188,11 +200,20 @@ class CausalLM:
         if self._launches_usable(ctx):
             stamp = self._launch_stamp(ctx)
             for view in self.entries:
+                self._offset(x, ctx, view)
                 self._run_block(self.blocks[view.block], x, ctx, view, stamp)
         else:
             for view in self.entries:
+                self._offset(x, ctx, view)
                 self.blocks[view.block].forward(x, ctx, view)
         return self._head(x, ctx)
+
+    def _offset(self, x, ctx, view) -> None:
+        """The vector that the schedule adds to the stream before this run, if any.  Sums that a
+        product has left in pieces stay owed: the vector is added to the stream's own part."""
+        offset = self.offsets.get(view.index)
+        if offset is not None:
+            self.ops.add_row_vector(x, offset[0], offset[1])
 
     MAX_KEPT_LAUNCHES = 256       # per scheduled run
 
@@ -277,6 +298,7 @@ class CausalLM:
         stamp = self._launch_stamp(ctx) if usable else None
         for view in self.entries:
             with r.range(f"block {view.index}"):
+                self._offset(x, ctx, view)
                 if usable:
                     self._run_block(self.blocks[view.block], x, ctx, view, stamp)
                 else:

@@ -2,7 +2,7 @@
 
 Kinds of library: ``core`` (embedding, norms, rotary + cache write, matrix
 products, sampling), ``attn_d<D>`` (attention for head size D; one per head
-size that a model needs), ``windowed_attention`` and ``linear_attention`` (mixers whose
+size that a model needs), ``windowed_attention``, ``linear_attention`` and ``routed_experts`` (parts whose
 sizes are run-time arguments; built when a model names them); beside them ``measure`` (stream and matrix-instruction loops for
 the benchmark's measured peaks) and the plain C++ references of the same operations,
 built with the host compiler for the tests.  A library's file name carries a hash of its sources
@@ -141,13 +141,15 @@ def attention_library(head_dim: int, force: bool = False) -> str:
     return _compile(f"attn_d{head_dim}", (ATTENTION_SOURCE,), (f"-DHEAD_DIM={head_dim}",), force)
 
 
-# Mixers with run-time sizes: one library each, whatever the head sizes of the model.
-MIXER_SOURCES = {"windowed_attention": "windowed_attention.hip", "linear_attention": "linear_attention.hip"}
+# Parts with run-time sizes: one library each, whatever the sizes of the model.
+MIXER_SOURCES = {"windowed_attention": "windowed_attention.hip", "linear_attention": "linear_attention.hip",
+                 "routed_experts": "routed_experts.hip"}
 
 
 def mixer_library(kind: str, force: bool = False) -> str:
     """``windowed_attention``: sliding window with a kept prefix and a sink term;
-    ``linear_attention``: the gated recurrence with a matrix state per head."""
+    ``linear_attention``: the gated recurrence with a matrix state per head; ``routed_experts``: a
+    feed-forward of many experts of which a row uses a few (choice, sorting, grouped products)."""
     return _compile(kind, (MIXER_SOURCES[kind],), (), force)
 
 
@@ -198,7 +200,8 @@ def reference_library(force: bool = False) -> str:
 
 def library(kind: str, parameter=None, force: bool = False) -> str:
     """The library a part names in ``kernel_libraries()``: ``("core", None)`` or
-    ``("attention", head_dim)``, ``("windowed_attention", None)``, ``("linear_attention", None)``."""
+    ``("attention", head_dim)``, ``("windowed_attention", None)``, ``("linear_attention", None)``,
+    ``("routed_experts", None)``."""
     if kind == "core":
         return core_library(force)
     if kind == "attention":

@@ -70,6 +70,22 @@ class PackedWeight:
         return self.data.element_size()
 
 
+class StackedWeight:
+    """Several matrices of equal shape ``[n, k]`` kept as one operand (``HipOps.prepare_stacked``):
+    ``data`` is the float32 tensor ``[members * n, k]`` or the packed bfloat16 matrix of ``members *
+    padded`` rows; a grouped product addresses member ``e`` by its first strip of rows."""
+
+    def __init__(self, data, members: int, n: int, padded: int, k: int):
+        self.data, self.members, self.n, self.padded, self.k = data, int(members), int(n), int(padded), int(k)
+        self.dtype = data.dtype
+
+    def numel(self) -> int:
+        return self.members * self.n * self.k
+
+    def element_size(self) -> int:
+        return self.data.element_size()
+
+
 class LaunchRecord:
     """The calls into the kernel libraries that a part made while it was recorded, so that
     the same part under the same conditions can make them again without its Python code:
@@ -143,7 +159,7 @@ class HipOps:
             self.device = torch.device("cuda", torch.cuda.current_device())
         self._core = self._load(build.core_library())
         self._declare_core()
-        if self._core.llmlab_abi_version() != 7:
+        if self._core.llmlab_abi_version() != 8:
             raise RuntimeError("kernel library and Python bindings disagree on the interface")
         self._attn: Dict[int, ctypes.CDLL] = {}
         self._mixer_libs: Dict[str, ctypes.CDLL] = {}
@@ -220,6 +236,10 @@ class HipOps:
         c.llmlab_layernorm_add.restype = _c_int
         c.llmlab_activation.argtypes = [_c_ptr, _c_ptr, _c_int, _c_int, _c_long, _c_ptr]
         c.llmlab_activation.restype = _c_int
+        c.llmlab_gate_heads.argtypes = [_c_ptr, _c_int, _c_ptr, _c_int, _c_int, _c_int, _c_ptr]
+        c.llmlab_gate_heads.restype = _c_int
+        c.llmlab_add_row_vector.argtypes = [_c_ptr, _c_ptr, _c_int, _c_int, _c_ptr]
+        c.llmlab_add_row_vector.restype = _c_int
         for fn in (c.llmlab_embed, c.llmlab_rmsnorm, c.llmlab_rope_kv_write, c.llmlab_rope_inplace,
                    c.llmlab_linear, c.llmlab_sample, c.llmlab_skinny_linear,
                    c.llmlab_linear_partials, c.llmlab_linear_qkv):
@@ -984,7 +1004,30 @@ class HipOps:
         self._call(self._core.llmlab_activation, self._ptr(x), self._ptr(out), _dt(out), self.ACTIVATIONS[kind],
                    x.numel(), self._stream())
 
-    # --------------------------------- mixers with run-time sizes (own libraries)
+    def gate_heads(self, out, gate, num_heads: int, head_dim: int, kind: str = "sigmoid") -> None:
+        """``out[r, h, :] *= sigmoid(gate[r, h])`` in place: ``out [rows, heads * head_dim]`` of a kernel
+        dtype, ``gate [rows, heads]`` float32; sigmoid and product in float32, one rounding."""
+        if kind != "sigmoid":
+            raise ValueError(f"gate_heads: unknown gate '{kind}'")
+        self._need(out, "mixer output")
+        self._need(gate, "head gates", torch.float32)
+        rows = out.shape[0]
+        if tuple(out.shape) != (rows, num_heads * head_dim) or tuple(gate.shape) != (rows, num_heads):
+            raise ValueError(f"gate_heads: output {tuple(out.shape)}, gates {tuple(gate.shape)} do not fit "
+                             f"{num_heads} heads of {head_dim}")
+        self._call(self._core.llmlab_gate_heads, self._ptr(out), _dt(out), self._ptr(gate), rows, int(num_heads),
+                   int(head_dim), self._stream())
+
+    def add_row_vector(self, x, table, row: int) -> None:
+        """``x[r, :] += table[row, :]`` for every row ``r`` of the float32 stream."""
+        self._need(x, "residual stream", torch.float32)
+        self._need(table, "offset table", torch.float32)
+        if table.dim() != 2 or table.shape[1] != x.shape[1] or not 0 <= row < table.shape[0]:
+            raise ValueError(f"add_row_vector: row {row} of a table {tuple(table.shape)} onto {tuple(x.shape)}")
+        self._call(self._core.llmlab_add_row_vector, self._ptr(x), table.data_ptr() + row * table.shape[1] * 4,
+                   x.shape[0], x.shape[1], self._stream())
+
+    # --------------------------------- parts with run-time sizes (own libraries)
     def _mixer_lib(self, kind: str) -> ctypes.CDLL:
         lib = self._mixer_libs.get(kind)
         if lib is None:
@@ -1017,9 +1060,78 @@ class HipOps:
                 lib.llmlab_gla_output.argtypes = [_c_ptr, _c_int, _c_int, _c_int, _c_int, _c_ptr, _c_float, _c_ptr,
                                                   _c_int, _c_int, _c_ptr, _c_int, _c_ptr]
                 lib.llmlab_gla_output.restype = _c_int
+            elif kind == "routed_experts":
+                lib.llmlab_moe_select.argtypes = [_c_ptr, _c_ptr, _c_int, _c_int, _c_int, _c_int, _c_int, _c_float,
+                                                  _c_ptr, _c_ptr, _c_ptr]
+                lib.llmlab_moe_select.restype = _c_int
+                lib.llmlab_moe_add_chosen.argtypes = [_c_ptr, _c_ptr, _c_int, _c_ptr, _c_ptr, _c_int, _c_int, _c_int,
+                                                      _c_int, _c_int, _c_ptr]
+                lib.llmlab_moe_add_chosen.restype = _c_int
             self._mixer_libs[kind] = lib
             self.loaded_libraries.append(lib._name)
         return lib
+
+    # ------------------------------------------------------- routed experts
+    def prepare_stacked(self, w: torch.Tensor, members: int) -> "StackedWeight":
+        """``members`` matrices of equal shape ``[n, k]``, one below the other in ``w``, as the product
+        kernels take them: float32 as they are; bfloat16 packed, every member padded to whole
+        strips of 16 rows, so that a member is a run of whole strips of the packed order."""
+        if w.dim() != 2 or members <= 0 or w.shape[0] % members:
+            raise ValueError(f"prepare_stacked: {tuple(w.shape)} is not {members} matrices of equal height")
+        n, k = w.shape[0] // members, w.shape[1]
+        if w.dtype == torch.float32:
+            return StackedWeight(self._need(w, "stacked weight"), members, n, n, k)
+        padded = (n + 15) // 16 * 16
+        if padded != n:
+            grown = torch.zeros((members, padded, k), dtype=w.dtype, device=w.device)
+            grown[:, :n] = w.view(members, n, k)
+            w = grown.view(members * padded, k)
+        return StackedWeight(self._prepare(w.contiguous()), members, n, padded, k)
+
+    def stacked_member(self, stacked: "StackedWeight", e: int):
+        """Member ``e`` as a weight operand of its own (a view, nothing is copied)."""
+        if not 0 <= e < stacked.members:
+            raise ValueError(f"a stack of {stacked.members} matrices has no member {e}")
+        if isinstance(stacked.data, PackedWeight):
+            per = self._core.llmlab_packed_elements(stacked.padded, stacked.k)
+            return PackedWeight(stacked.data.data[e * per:(e + 1) * per], stacked.n, stacked.k)
+        return stacked.data[e * stacked.n:(e + 1) * stacked.n]
+
+    def moe_grouped(self, dtype) -> bool:
+        """Whether the experts of this dtype run as grouped products over rows sorted by expert."""
+        return False
+
+    def moe_select(self, logits, correction, groups: int, groups_keep: int, scale: float, chosen, weights) -> None:
+        """Per row of the router's float32 ``logits [rows, outputs]``: scores ``softmax(logits)``; choice
+        values ``score + correction``; the outputs form ``groups`` equal groups of neighbours of which
+        the ``groups_keep`` with the largest best choice value stay; ``chosen [rows, top]`` (int32) are
+        the outputs with the largest choice values among those (ties: the smaller index), ``weights
+        [rows, top]`` their scores times ``scale``."""
+        lib = self._mixer_lib("routed_experts")
+        self._need(logits, "router logits", torch.float32)
+        self._need(correction, "router correction", torch.float32)
+        self._need(chosen, "chosen experts", torch.int32)
+        self._need(weights, "expert weights", torch.float32)
+        rows, outputs = logits.shape
+        top = chosen.shape[1]
+        if correction.numel() != outputs or tuple(chosen.shape) != (rows, top) or tuple(weights.shape) != (rows, top):
+            raise ValueError("moe_select: shapes do not fit")
+        self._call(lib.llmlab_moe_select, self._ptr(logits), self._ptr(correction), rows, outputs, int(groups),
+                   int(groups_keep), top, float(scale), self._ptr(chosen), self._ptr(weights), self._stream(), lib=lib)
+
+    def moe_add_chosen(self, resid, src, chosen, weights, first: int, last: int) -> None:
+        """``resid[r] += w_r * src[r]`` with ``w_r`` the sum of ``weights[r, k]`` over the ``k`` whose
+        ``chosen[r, k]`` lies in ``[first, last)``; rows that chose none of them are left alone."""
+        lib = self._mixer_lib("routed_experts")
+        self._need(resid, "residual stream", torch.float32)
+        self._need(src, "expert output")
+        self._need(chosen, "chosen experts", torch.int32)
+        self._need(weights, "expert weights", torch.float32)
+        rows, hidden = resid.shape
+        if tuple(src.shape) != (rows, hidden) or chosen.shape[0] != rows or tuple(weights.shape) != tuple(chosen.shape):
+            raise ValueError("moe_add_chosen: shapes do not fit")
+        self._call(lib.llmlab_moe_add_chosen, self._ptr(resid), self._ptr(src), _dt(src), self._ptr(chosen),
+                   self._ptr(weights), rows, chosen.shape[1], int(first), int(last), hidden, self._stream(), lib=lib)
 
     def check_windowed_attention_sizes(self, num_heads, num_kv_heads, key_dim, value_dim, dtype) -> None:
         if num_heads % num_kv_heads:

@@ -6,4 +6,5 @@ from .positions import RotaryEmbedding, NoPosition
 from .attention import GQAAttention, WindowedSinkAttention
 from .linear_attention import GatedLinearAttention
 from .feed_forward import SwiGLU, DenseFeedForward, interleave_gate_up
+from .experts import RoutedExperts
 from .blocks import PreNormBlock, SublayerNormBlock, TokenEmbedding, LinearHead

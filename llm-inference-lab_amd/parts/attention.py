@@ -27,17 +27,30 @@ class GQAAttention(Mixer):
     cache write engine.rs:1072-1082, scores/softmax
     rust/engine/src/runner/model/qwen2/kernels.rs:702-853, output projection and
     residual engine.rs:1225-1233.  The window is not in the reference (it
-    rejects ``use_sliding_window``, engine.rs:262)."""
+    rejects ``use_sliding_window``, engine.rs:262).
+
+    ``values_from_keys``: the layer has no value projection; its values are its keys as
+    projected (bias added), before the position encoding turns them.  ``output_gate="sigmoid"``:
+    one more projection of the layer's input, a single number per head (``gate_weight [heads,
+    hidden]``, no bias); head ``h``'s output is multiplied by ``sigmoid`` of its number before the
+    output projection."""
 
     takes_normed_input = True
+    OUTPUT_GATES = (None, "sigmoid")
 
     def __init__(self, hidden_size: int, num_heads: int, num_kv_heads: int, head_dim: int,
                  position: Optional[PartSpec], tensors: Dict[str, str], qkv_bias: bool = True,
                  out_bias: bool = False, window: Optional[int] = None,
-                 scale: Optional[float] = None):
+                 scale: Optional[float] = None, values_from_keys: bool = False,
+                 output_gate: Optional[str] = None):
         super().__init__(tensors)
         if num_heads % num_kv_heads:
             raise ValueError(f"{num_heads} heads are not a multiple of {num_kv_heads} kv heads")
+        if output_gate not in self.OUTPUT_GATES:
+            raise ValueError(f"an output gate is one of {self.OUTPUT_GATES}, got {output_gate!r}")
+        self.values_from_keys = bool(values_from_keys)
+        self.output_gate = output_gate
+        self.w_gate = None
         self.hidden_size = int(hidden_size)
         self.num_heads = int(num_heads)
         self.num_kv_heads = int(num_kv_heads)
@@ -63,13 +76,17 @@ class GQAAttention(Mixer):
         specs = {
             t["q_weight"]: TensorSpec((self.q_size, h), MATRIX),
             t["k_weight"]: TensorSpec((self.kv_size, h), MATRIX),
-            t["v_weight"]: TensorSpec((self.kv_size, h), MATRIX),
             t["o_weight"]: TensorSpec((h, self.q_size), MATRIX),
         }
+        if not self.values_from_keys:
+            specs[t["v_weight"]] = TensorSpec((self.kv_size, h), MATRIX)
+        if self.output_gate:
+            specs[t["gate_weight"]] = TensorSpec((self.num_heads, h), MATRIX)
         if self.qkv_bias:
             specs[t["q_bias"]] = TensorSpec((self.q_size,), VECTOR)
             specs[t["k_bias"]] = TensorSpec((self.kv_size,), VECTOR)
-            specs[t["v_bias"]] = TensorSpec((self.kv_size,), VECTOR)
+            if not self.values_from_keys:
+                specs[t["v_bias"]] = TensorSpec((self.kv_size,), VECTOR)
         if self.out_bias:
             specs[t["o_bias"]] = TensorSpec((h,), VECTOR)
         if self.position is not None:
@@ -82,13 +99,29 @@ class GQAAttention(Mixer):
         ops.check_product_sizes(self.hidden_size, dtype, "attention projections (hidden size)")
         ops.check_product_sizes(self.q_size, dtype, "attention output projection (heads * head size)")
         t = self.tensor_names
+        # The order in which the position encoding wants the channels of the query and key heads
+        # (scores do not depend on it; values and the output projection keep the file's order).
+        order = self.position.channel_order() if self.position is not None else None
+
+        def heads_in_order(x, heads):
+            if order is None:
+                return x
+            index = torch.tensor(order, device=x.device)
+            return x.unflatten(0, (heads, self.head_dim)).index_select(1, index).flatten(0, 1)
+        # Values that are the keys before they turn: the key rows once more, in the file's order,
+        # in the value rows' place, so that the product and its epilogues stay as they are.
+        value = "k" if self.values_from_keys else "v"
         # One projection instead of three: the rows of Wq, Wk, Wv stacked.
-        self.w_qkv = ops.prepare_weight(torch.cat([tensors[t["q_weight"]], tensors[t["k_weight"]],
-                                                   tensors[t["v_weight"]]], dim=0).contiguous())
+        self.w_qkv = ops.prepare_weight(torch.cat([heads_in_order(tensors[t["q_weight"]], self.num_heads),
+                                                   heads_in_order(tensors[t["k_weight"]], self.num_kv_heads),
+                                                   tensors[t[value + "_weight"]]], dim=0).contiguous())
         if self.qkv_bias:
-            parts = [tensors[t["q_bias"]], tensors[t["k_bias"]], tensors[t["v_bias"]]]
+            parts = [heads_in_order(tensors[t["q_bias"]], self.num_heads),
+                     heads_in_order(tensors[t["k_bias"]], self.num_kv_heads), tensors[t[value + "_bias"]]]
             kept = parts[0].dtype if all(p.dtype == parts[0].dtype for p in parts) else torch.float32
             self.b_qkv = torch.cat([p.to(kept) for p in parts]).contiguous()
+        if self.output_gate:
+            self.w_gate = ops.prepare_weight(tensors[t["gate_weight"]].contiguous())
         self.w_o = ops.prepare_weight(tensors[t["o_weight"]].contiguous())
         self.b_o = tensors[t["o_bias"]].contiguous() if self.out_bias else None
         if self.position is not None:
@@ -109,6 +142,7 @@ class GQAAttention(Mixer):
                 and not ops.pieces_too_large_to_read_per_block(getattr(ctx, "pending", None)))
         rms = h.rms(accept_pending=True) if fuse else None
         pending = None
+        gate = ctx.scratch("attention.gate", (rows, self.num_heads), torch.float32) if self.output_gate else None
         if rms is not None:
             # few rows: norm, the three projections, bias, rotation and the cache
             # write are one kernel
@@ -119,6 +153,8 @@ class GQAAttention(Mixer):
             ops.fused_norm_qkv(rms[0], rms[2], rms[3], self.w_qkv, self.b_qkv, self.num_heads,
                                self.num_kv_heads, self.head_dim, table, ctx.positions, ctx.row_req,
                                group.block_table, group.page_size, k_cache, v_cache, q, pending=pending)
+            if gate is not None:           # (the gate reads the same normed rows: norm and product in one kernel too)
+                ops.fused_norm_logits(rms[0], None, rms[2], rms[3], self.w_gate, gate, pending=pending)
         elif (ops.can_fuse_qkv_rope(rows, self.dtype, self.head_dim, self.q_size + 2 * self.kv_size,
                                     self.hidden_size)
               and (self.position is None or table is not None)):
@@ -142,6 +178,8 @@ class GQAAttention(Mixer):
             ops.rope_kv_write(q, self.num_heads, self.num_kv_heads, self.head_dim, table,
                               ctx.positions, ctx.row_req, group.block_table, group.page_size,
                               k_cache, v_cache)
+        if gate is not None and rms is None:
+            ops.linear_logits(h, self.w_gate, gate)
         out = ctx.scratch("attention.out", (rows, self.q_size), self.dtype)
 
         prepare = getattr(ops, "prepare_attention", None)
@@ -169,6 +207,8 @@ class GQAAttention(Mixer):
             live(attend)
         else:
             attend()
+        if gate is not None:
+            ops.gate_heads(out, gate, self.num_heads, self.head_dim, self.output_gate)
         if pending is not None:
             ops.linear_residual(out, self.w_o, residual, self.b_o, pending=pending)
             ctx.pending = None
@@ -211,7 +251,7 @@ class GQAAttention(Mixer):
 
     def weight_bytes(self):
         total = 0
-        for w in (self.w_qkv, self.b_qkv, self.w_o, self.b_o):
+        for w in (self.w_qkv, self.b_qkv, self.w_o, self.b_o, self.w_gate):
             if w is not None:
                 total += w.numel() * w.element_size()
         return total

@@ -219,6 +219,11 @@ class PositionEncoding(Part):
         that the fused projection epilogue can apply; None otherwise."""
         return None
 
+    def channel_order(self):
+        """None, or the order in which a mixer lays out the channels of every query and key head
+        (place -> channel of the model file) for ``rotary_table()`` to apply."""
+        return None
+
     def apply(self, q: torch.Tensor, k: torch.Tensor, positions: torch.Tensor) -> None:
         """Encode positions into ``q [rows, heads, dim]`` and ``k`` in place."""
         raise NotImplementedError

@@ -18,17 +18,20 @@ class PreNormBlock(Block):
     Arrangement: rust/engine/src/runner/model/qwen2/engine.rs:1065-1122 (layer
     loop), 1140-1147 and 1234-1241 (norm before each sublayer)."""
 
-    def __init__(self, hidden_size: int, norm1: PartSpec, mixer: PartSpec, norm2: PartSpec,
-                 feed_forward: PartSpec, tensors: Dict[str, str] = None):
+    def __init__(self, hidden_size: int, norm1: PartSpec, mixer: PartSpec, norm2: PartSpec = None,
+                 feed_forward: PartSpec = None, tensors: Dict[str, str] = None):
         super().__init__(tensors)
+        if (feed_forward is None) != (norm2 is None):
+            raise ValueError("a feed-forward and its norm come together")
         self.hidden_size = int(hidden_size)
         self.norm1 = build_part("norm", norm1)
         self.mixer = build_part("mixer", mixer)
-        self.norm2 = build_part("norm", norm2)
-        self.feed_forward = build_part("feed_forward", feed_forward)
+        # (a layer may be its mixer alone)
+        self.norm2 = build_part("norm", norm2) if norm2 is not None else None
+        self.feed_forward = build_part("feed_forward", feed_forward) if feed_forward is not None else None
 
     def parts(self):
-        return [self.norm1, self.mixer, self.norm2, self.feed_forward]
+        return [p for p in (self.norm1, self.mixer, self.norm2, self.feed_forward) if p is not None]
 
     def mixer_part(self):
         return self.mixer
@@ -47,6 +50,8 @@ class PreNormBlock(Block):
     def forward(self, residual, ctx, entry):
         h = NormedInput(self.norm1, residual, ctx, "block.normed", self.dtype)
         self.mixer.forward(h if self.mixer.takes_normed_input else h.tensor(), residual, ctx, entry)
+        if self.feed_forward is None:
+            return
         h = NormedInput(self.norm2, residual, ctx, "block.normed", self.dtype)
         self.feed_forward.forward(h if self.feed_forward.takes_normed_input else h.tensor(),
                                   residual, ctx)

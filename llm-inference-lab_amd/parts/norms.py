@@ -5,7 +5,7 @@ from typing import Dict, Optional
 
 import torch
 
-from ..weights.loader import TensorSpec, VECTOR, INIT_NORM
+from ..weights.loader import TensorSpec, VECTOR, INIT_NORM, INIT_NORMAL
 from .base import Norm
 from .registry import register_part
 
@@ -16,23 +16,29 @@ class RMSNorm(Norm):
 
     Formula: rust/engine/src/runner/model/qwen2/kernels.rs:546-582 (the
     reference rounds once more, before the weight product; in float32 the two
-    are the same).  ``size`` and ``eps`` come from the caller."""
+    are the same).  ``size`` and ``eps`` come from the caller.  ``weight_offset``: the stored
+    tensor is the scale less this constant (a weight kept around zero has ``weight_offset=1``:
+    ``w = 1 + stored``); the sum is taken once, in float32, when the part is bound."""
 
     folds_pending = True
     keeps_launches = True
 
-    def __init__(self, size: int, eps: float, tensors: Dict[str, str]):
+    def __init__(self, size: int, eps: float, tensors: Dict[str, str], weight_offset: float = 0.0):
         super().__init__(tensors)
         self.size = int(size)
         self.eps = float(eps)
+        self.weight_offset = float(weight_offset)
         self.weight: Optional[torch.Tensor] = None
 
     def tensor_specs(self):
-        return {self.tensor_names["weight"]: TensorSpec((self.size,), VECTOR, INIT_NORM)}
+        return {self.tensor_names["weight"]: TensorSpec((self.size,), VECTOR,
+                                                        INIT_NORMAL if self.weight_offset else INIT_NORM)}
 
     def bind(self, tensors, ops, dtype):
         super().bind(tensors, ops, dtype)
         self.weight = tensors[self.tensor_names["weight"]].contiguous()
+        if self.weight_offset:
+            self.weight = (self.weight.float() + self.weight_offset).contiguous()
 
     def forward(self, x, out, rows=None, pending=None):
         if pending is None:

@@ -15,21 +15,42 @@ class RotaryEmbedding(PositionEncoding):
     hi*cos + lo*sin]``; angles, sines and cosines in float32.
 
     Formula: rust/engine/src/runner/model/qwen2/kernels.rs:587-631; frequency
-    table: rust/engine/src/runner/model/qwen2/engine.rs:304-306."""
+    table: rust/engine/src/runner/model/qwen2/engine.rs:304-306.
 
-    def __init__(self, dim: int, theta: float, tensors: Optional[Dict[str, str]] = None):
+    ``rotary_dim`` (default: all of ``dim``): only the first ``rotary_dim`` channels of a head
+    turn, channel ``i`` with channel ``i + rotary_dim/2`` by ``position * theta^(-2i/rotary_dim)``,
+    the others pass unchanged.  The kernels turn channel ``j`` of a head with channel ``j +
+    dim/2``, so the part names the order in which a mixer has to lay out the channels of its
+    query and key heads (``channel_order()``: scores do not depend on a common order of both)
+    and gives the channels that do not turn the frequency 0: an angle of exactly 0, whose cosine
+    is 1 and whose sine is 0."""
+
+    def __init__(self, dim: int, theta: float, tensors: Optional[Dict[str, str]] = None,
+                 rotary_dim: Optional[int] = None):
         super().__init__(tensors)
-        if dim % 2:
-            raise ValueError(f"rotary dimension {dim} must be even")
         self.dim = int(dim)
+        self.rotary_dim = self.dim if rotary_dim is None else int(rotary_dim)
+        if self.dim % 2 or self.rotary_dim % 2 or not 0 <= self.rotary_dim <= self.dim:
+            raise ValueError(f"a head of {dim} channels of which {self.rotary_dim} turn: both must be even")
         self.theta = float(theta)
         self.inv_freq: Optional[torch.Tensor] = None
 
     def bind(self, tensors, ops, dtype):
         super().bind(tensors, ops, dtype)
-        exponent = torch.arange(0, self.dim, 2, dtype=torch.float64) / self.dim
-        self.inv_freq = (1.0 / (torch.tensor(self.theta, dtype=torch.float64) ** exponent)
-                         ).to(torch.float32).to(ops.device)
+        exponent = torch.arange(0, self.rotary_dim, 2, dtype=torch.float64) / max(self.rotary_dim, 1)
+        freq = torch.zeros(self.dim // 2, dtype=torch.float64)
+        freq[:self.rotary_dim // 2] = 1.0 / (torch.tensor(self.theta, dtype=torch.float64) ** exponent)
+        self.inv_freq = freq.to(torch.float32).to(ops.device)
+
+    def channel_order(self):
+        """``order[j]``: which channel of a head, as the model file has it, goes to place ``j`` so that
+        the pairs ``(j, j + dim/2)`` are the pairs that turn together; None if that is the file's
+        own order."""
+        if self.rotary_dim == self.dim:
+            return None
+        half, rest = self.rotary_dim // 2, (self.dim - self.rotary_dim) // 2
+        still = list(range(self.rotary_dim, self.dim))
+        return (list(range(half)) + still[:rest]) + (list(range(half, 2 * half)) + still[rest:])
 
     keeps_launches = True      # (the frequency table goes to the kernels; ``apply`` depends on the rows only)
 

@@ -59,7 +59,8 @@ class EmuOps:
                 "add_pending", "linear_logits", "linear_swiglu", "fused_norm_qkv", "qkv_rope_cache",
                 "fused_norm_swiglu", "fused_norm_logits", "rope_inplace", "rope_kv_write",
                 "paged_attention", "argmax", "sample", "layernorm", "layernorm_add", "activation",
-                "project_norm_write", "sink_window_attention", "gla_decay", "gla_scan", "gla_output")
+                "project_norm_write", "sink_window_attention", "gla_decay", "gla_scan", "gla_output",
+                "gate_heads", "add_row_vector", "moe_select", "moe_add_chosen")
 
     def __init__(self, device="cpu", fuse=True):
         self.device = torch.device(device)
@@ -362,6 +363,60 @@ class EmuOps:
 
     def release_shared(self):
         pass
+
+    # --------------------------------------------- gates, offsets, routed experts
+    def gate_heads(self, out, gate, num_heads, head_dim, kind="sigmoid"):
+        """``out[r, h, :] *= sigmoid(gate[r, h])``, the product in float32, one rounding."""
+        self._count("gate_heads")
+        assert kind == "sigmoid"
+        v = out.float().view(out.shape[0], num_heads, head_dim) * torch.sigmoid(gate.float())[:, :, None]
+        out.copy_(v.view(out.shape).to(out.dtype))
+
+    def add_row_vector(self, x, table, row):
+        self._count("add_row_vector")
+        x += table[row].float()
+
+    def prepare_stacked(self, w, members):
+        return w.view(members, w.shape[0] // members, w.shape[1])
+
+    def stacked_member(self, stacked, e):
+        return stacked[e]
+
+    def moe_grouped(self, dtype):
+        return False
+
+    def moe_select(self, logits, correction, groups, groups_keep, scale, chosen, weights):
+        """Per row: softmax of the logits, the choice value (score + correction), the kept groups by
+        their best choice value, the ``top`` best of their members; ties to the smaller index."""
+        self._count("moe_select")
+        rows, outputs = logits.shape
+        top = chosen.shape[1]
+        z = logits.float()
+        e = torch.exp(z - z.max(-1, keepdim=True).values)
+        s = e / e.sum(-1, keepdim=True)
+        c = s + correction.float()
+        per = outputs // groups
+        best = c.view(rows, groups, per).max(-1).values
+        allowed = torch.zeros(rows, groups, dtype=torch.bool)
+        left = best.clone()
+        for _ in range(groups_keep):
+            g = torch.argmax(left, dim=-1)            # (the first of equal ones)
+            allowed[torch.arange(rows), g] = True
+            left[torch.arange(rows), g] = -float("inf")
+        c = torch.where(allowed[:, :, None].expand(rows, groups, per).reshape(rows, outputs), c,
+                        torch.full_like(c, -float("inf")))
+        for k in range(top):
+            e_k = torch.argmax(c, dim=-1)
+            chosen[:, k] = e_k.to(torch.int32)
+            weights[:, k] = s[torch.arange(rows), e_k] * scale
+            c[torch.arange(rows), e_k] = -float("inf")
+
+    def moe_add_chosen(self, resid, src, chosen, weights, first, last):
+        """``resid[r] += sum over k with first <= chosen[r, k] < last of weights[r, k] * src[r]``."""
+        self._count("moe_add_chosen")
+        hit = (chosen >= first) & (chosen < last)
+        w = (weights * hit).sum(-1, keepdim=True)
+        resid += w * src.float()
 
     def _normed(self, x, rows_index, norm_w, eps, n, pending=None):
         v = x.float() + self._owed(pending)
