@@ -33,7 +33,11 @@ class GQAAttention(Mixer):
     projected (bias added), before the position encoding turns them.  ``output_gate="sigmoid"``:
     one more projection of the layer's input, a single number per head (``gate_weight [heads,
     hidden]``, no bias); head ``h``'s output is multiplied by ``sigmoid`` of its number before the
-    output projection."""
+    output projection.
+
+    The kernels take heads whose size is a multiple of 16: a head of another size is laid out
+    with zeros behind its channels (zero rows of the projections, zero columns of the output
+    projection), which changes no score and no output."""
 
     takes_normed_input = True
     OUTPUT_GATES = (None, "sigmoid")
@@ -54,12 +58,14 @@ class GQAAttention(Mixer):
         self.hidden_size = int(hidden_size)
         self.num_heads = int(num_heads)
         self.num_kv_heads = int(num_kv_heads)
-        self.head_dim = int(head_dim)
+        self.file_head_dim = int(head_dim)                       # a head as the model file has it
+        self.head_dim = (self.file_head_dim + 15) // 16 * 16     # and as the kernels see it
         self.qkv_bias = bool(qkv_bias)
         self.out_bias = bool(out_bias)
         self.window = None if window is None else int(window)
-        self.scale = float(scale) if scale is not None else 1.0 / math.sqrt(self.head_dim)
-        self.position = build_part("position", position) if position is not None else None
+        self.scale = float(scale) if scale is not None else 1.0 / math.sqrt(self.file_head_dim)
+        padded = dict(padded_dim=self.head_dim) if self.head_dim != self.file_head_dim else {}
+        self.position = build_part("position", position, **padded) if position is not None else None
         self.w_qkv = self.b_qkv = self.w_o = self.b_o = None
 
     # sizes
@@ -73,20 +79,21 @@ class GQAAttention(Mixer):
 
     def tensor_specs(self):
         t, h = self.tensor_names, self.hidden_size
+        q_size, kv_size = self.num_heads * self.file_head_dim, self.num_kv_heads * self.file_head_dim
         specs = {
-            t["q_weight"]: TensorSpec((self.q_size, h), MATRIX),
-            t["k_weight"]: TensorSpec((self.kv_size, h), MATRIX),
-            t["o_weight"]: TensorSpec((h, self.q_size), MATRIX),
+            t["q_weight"]: TensorSpec((q_size, h), MATRIX),
+            t["k_weight"]: TensorSpec((kv_size, h), MATRIX),
+            t["o_weight"]: TensorSpec((h, q_size), MATRIX),
         }
         if not self.values_from_keys:
-            specs[t["v_weight"]] = TensorSpec((self.kv_size, h), MATRIX)
+            specs[t["v_weight"]] = TensorSpec((kv_size, h), MATRIX)
         if self.output_gate:
             specs[t["gate_weight"]] = TensorSpec((self.num_heads, h), MATRIX)
         if self.qkv_bias:
-            specs[t["q_bias"]] = TensorSpec((self.q_size,), VECTOR)
-            specs[t["k_bias"]] = TensorSpec((self.kv_size,), VECTOR)
+            specs[t["q_bias"]] = TensorSpec((q_size,), VECTOR)
+            specs[t["k_bias"]] = TensorSpec((kv_size,), VECTOR)
             if not self.values_from_keys:
-                specs[t["v_bias"]] = TensorSpec((self.kv_size,), VECTOR)
+                specs[t["v_bias"]] = TensorSpec((kv_size,), VECTOR)
         if self.out_bias:
             specs[t["o_bias"]] = TensorSpec((h,), VECTOR)
         if self.position is not None:
@@ -102,27 +109,37 @@ class GQAAttention(Mixer):
         # The order in which the position encoding wants the channels of the query and key heads
         # (scores do not depend on it; values and the output projection keep the file's order).
         order = self.position.channel_order() if self.position is not None else None
+        d, dk = self.file_head_dim, self.head_dim
+        plain = list(range(d)) + [-1] * (dk - d)          # the file's order, zeros behind
 
-        def heads_in_order(x, heads):
-            if order is None:
+        def heads_in_order(x, heads, order=order):
+            """Rows (or entries) of ``heads`` heads of ``d`` channels -> heads of ``dk`` places."""
+            order = plain if order is None else order
+            if order == list(range(d)):
                 return x
-            index = torch.tensor(order, device=x.device)
-            return x.unflatten(0, (heads, self.head_dim)).index_select(1, index).flatten(0, 1)
+            per_head = x.unflatten(0, (heads, d))
+            per_head = torch.cat([per_head, torch.zeros_like(per_head[:, :1])], dim=1)     # place -1: a zero
+            index = torch.tensor([d if c < 0 else c for c in order], device=x.device)
+            return per_head.index_select(1, index).flatten(0, 1)
         # Values that are the keys before they turn: the key rows once more, in the file's order,
         # in the value rows' place, so that the product and its epilogues stay as they are.
         value = "k" if self.values_from_keys else "v"
         # One projection instead of three: the rows of Wq, Wk, Wv stacked.
         self.w_qkv = ops.prepare_weight(torch.cat([heads_in_order(tensors[t["q_weight"]], self.num_heads),
                                                    heads_in_order(tensors[t["k_weight"]], self.num_kv_heads),
-                                                   tensors[t[value + "_weight"]]], dim=0).contiguous())
+                                                   heads_in_order(tensors[t[value + "_weight"]], self.num_kv_heads,
+                                                                  None)], dim=0).contiguous())
         if self.qkv_bias:
             parts = [heads_in_order(tensors[t["q_bias"]], self.num_heads),
-                     heads_in_order(tensors[t["k_bias"]], self.num_kv_heads), tensors[t[value + "_bias"]]]
+                     heads_in_order(tensors[t["k_bias"]], self.num_kv_heads),
+                     heads_in_order(tensors[t[value + "_bias"]], self.num_kv_heads, None)]
             kept = parts[0].dtype if all(p.dtype == parts[0].dtype for p in parts) else torch.float32
             self.b_qkv = torch.cat([p.to(kept) for p in parts]).contiguous()
         if self.output_gate:
             self.w_gate = ops.prepare_weight(tensors[t["gate_weight"]].contiguous())
-        self.w_o = ops.prepare_weight(tensors[t["o_weight"]].contiguous())
+        # (the heads' outputs arrive in the values' order: the columns of the output projection
+        # are its own, with zero columns behind every head)
+        self.w_o = ops.prepare_weight(heads_in_order(tensors[t["o_weight"]].t(), self.num_heads, None).t().contiguous())
         self.b_o = tensors[t["o_bias"]].contiguous() if self.out_bias else None
         if self.position is not None:
             self.position.bind(tensors, ops, dtype)

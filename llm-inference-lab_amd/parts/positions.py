@@ -23,34 +23,41 @@ class RotaryEmbedding(PositionEncoding):
     dim/2``, so the part names the order in which a mixer has to lay out the channels of its
     query and key heads (``channel_order()``: scores do not depend on a common order of both)
     and gives the channels that do not turn the frequency 0: an angle of exactly 0, whose cosine
-    is 1 and whose sine is 0."""
+    is 1 and whose sine is 0.  ``padded_dim``: the mixer's kernels work on heads of that many
+    channels (the head's own, then zeros); the table and the order are made for those."""
 
     def __init__(self, dim: int, theta: float, tensors: Optional[Dict[str, str]] = None,
-                 rotary_dim: Optional[int] = None):
+                 rotary_dim: Optional[int] = None, padded_dim: Optional[int] = None):
         super().__init__(tensors)
         self.dim = int(dim)
         self.rotary_dim = self.dim if rotary_dim is None else int(rotary_dim)
-        if self.dim % 2 or self.rotary_dim % 2 or not 0 <= self.rotary_dim <= self.dim:
-            raise ValueError(f"a head of {dim} channels of which {self.rotary_dim} turn: both must be even")
+        self.padded_dim = self.dim if padded_dim is None else int(padded_dim)
+        if self.rotary_dim % 2 or not 0 <= self.rotary_dim <= self.dim:
+            raise ValueError(f"a head of {dim} channels of which {self.rotary_dim} turn in pairs")
+        if self.padded_dim % 2 or self.padded_dim < self.dim + self.dim % 2:
+            raise ValueError(f"heads of {dim} channels do not fit an even {self.padded_dim}")
         self.theta = float(theta)
         self.inv_freq: Optional[torch.Tensor] = None
 
     def bind(self, tensors, ops, dtype):
         super().bind(tensors, ops, dtype)
         exponent = torch.arange(0, self.rotary_dim, 2, dtype=torch.float64) / max(self.rotary_dim, 1)
-        freq = torch.zeros(self.dim // 2, dtype=torch.float64)
+        freq = torch.zeros(self.padded_dim // 2, dtype=torch.float64)
         freq[:self.rotary_dim // 2] = 1.0 / (torch.tensor(self.theta, dtype=torch.float64) ** exponent)
         self.inv_freq = freq.to(torch.float32).to(ops.device)
 
     def channel_order(self):
-        """``order[j]``: which channel of a head, as the model file has it, goes to place ``j`` so that
-        the pairs ``(j, j + dim/2)`` are the pairs that turn together; None if that is the file's
-        own order."""
-        if self.rotary_dim == self.dim:
+        """``order[j]``: which channel of a head, as the model file has it, goes to place ``j`` (-1: a
+        zero) so that the pairs ``(j, j + padded_dim/2)`` are the pairs that turn together; None if
+        that is the file's own order."""
+        if self.rotary_dim == self.dim == self.padded_dim:
             return None
-        half, rest = self.rotary_dim // 2, (self.dim - self.rotary_dim) // 2
+        half, places = self.rotary_dim // 2, self.padded_dim // 2
         still = list(range(self.rotary_dim, self.dim))
-        return (list(range(half)) + still[:rest]) + (list(range(half, 2 * half)) + still[rest:])
+        first = (len(still) + 1) // 2
+        low = list(range(half)) + still[:first]
+        high = list(range(half, 2 * half)) + still[first:]
+        return low + [-1] * (places - len(low)) + high + [-1] * (places - len(high))
 
     keeps_launches = True      # (the frequency table goes to the kernels; ``apply`` depends on the rows only)
 

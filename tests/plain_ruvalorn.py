@@ -5,8 +5,6 @@ no batching.  ``weights`` maps tensor names to float64 tensors, ``cfg`` is the d
 ``config.json``.  Notation: ``n`` tokens, width ``w``; a linear map stored ``[out, in]`` is applied
 as ``x @ W.T``.
 """
-import math
-
 import torch
 
 
@@ -40,6 +38,11 @@ def rotate(x, positions, dims, base):
     return out
 
 
+def gate_heads(out, gate_logits):
+    """``out [n, heads, d]`` times one sigmoid per token and head."""
+    return out * torch.sigmoid(gate_logits)[:, :, None]
+
+
 def visible(i, j, window):
     """Whether the query at position i reads the key at position j."""
     return 0 <= i - j and (window is None or i - j < window)
@@ -58,7 +61,6 @@ def attention(h, weights, prefix, m):
     q = rotate(q, positions, rot.get("dims", 0), rot.get("base", 1.0))
     k = rotate(k, positions, rot.get("dims", 0), rot.get("base", 1.0))
     window = (m.get("mask") or {}).get("size")
-    gate = torch.sigmoid(h @ weights[prefix + "g"].T)            # [n, heads]
     out = torch.zeros(n, heads, d, dtype=h.dtype)
     for head in range(heads):
         g = head // (heads // groups)
@@ -66,7 +68,8 @@ def attention(h, weights, prefix, m):
             seen = [j for j in range(n) if visible(i, j, window)]
             scores = (k[seen, g] @ q[i, head]) * m["scale"]
             p = torch.softmax(scores, 0)
-            out[i, head] = (p @ values[seen, g]) * gate[i, head]
+            out[i, head] = p @ values[seen, g]
+    out = gate_heads(out, h @ weights[prefix + "g"].T)
     return out.reshape(n, heads * d) @ weights[prefix + "o"].T
 
 
