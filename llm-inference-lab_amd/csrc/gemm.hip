@@ -72,6 +72,13 @@ struct EpiArgs {
   int table_stride, page_size, nq, nkv, d;
   // STORE only: 1 = the sum goes through max(z, 0)^2 (in float32) before it is rounded
   int act;
+  // Grouped products (several matrices of equal shape, one below the other in W; every tile of
+  // rows belongs to one of them): g_tile[tile of rows] is the tile's matrix (-1: the tile is
+  // empty), g_w_stride the packed elements of one matrix, g_rows (may be null) the row of x that
+  // row m of the product reads (-1: none; such rows' results land in rows nobody reads).
+  const int* g_tile;
+  const int* g_rows;
+  size_t g_w_stride;
 };
 
 __device__ __forceinline__ float relu2_f(float z) {
@@ -286,7 +293,7 @@ __device__ __forceinline__ void tile_epilogue(const float* Cs, const EpiArgs& e,
 }
 
 // ============================================================ bf16, tiled
-template <int BM, int BN, int BK, int WM, int WN, int EPI>
+template <int BM, int BN, int BK, int WM, int WN, int EPI, bool GROUPED = false>
 __global__ __launch_bounds__(64 * WM * WN) void gemm_bf16_tiled(const bf16_t* __restrict__ A,
                                                         const bf16_t* __restrict__ W, EpiArgs e, int M,
                                                         int N, int K) {
@@ -323,6 +330,11 @@ __global__ __launch_bounds__(64 * WM * WN) void gemm_bf16_tiled(const bf16_t* __
   }
   const int m0 = by * BM, n0 = bx * BN;
   const int c = lane & 15, g = lane >> 4;
+  if constexpr (GROUPED) {
+    const int member = e.g_tile[by];       // (the same for the whole block: all leave together)
+    if (member < 0) return;
+    W += (size_t)member * e.g_w_stride;
+  }
 
   // QKV: what the epilogue needs from global memory per row of the tile (position, and the
   // page of that position for the tiles that hold k or v heads) and per column (bias,
@@ -366,11 +378,19 @@ __global__ __launch_bounds__(64 * WM * WN) void gemm_bf16_tiled(const bf16_t* __
   // stores.  W is packed in fragment order: the 64 columns of a strip of 16 rows
   // are consecutive memory (1 KB per 32 columns), a thread reading 16 bytes of it.
   const int T = (K + 31) >> 5, nstrips = (N + 15) >> 4;
+  int gathered[GROUPED ? A_CHUNKS : 1];      // GROUPED: the rows of x this thread's pieces come from
+  if constexpr (GROUPED) {
+#pragma unroll
+    for (int i = 0; i < A_CHUNKS; ++i) {
+      const int m = min(m0 + (tid + i * NT) / KCH, M - 1);
+      gathered[i] = e.g_rows ? max(e.g_rows[m], 0) : m;
+    }
+  }
   auto fetch = [&](int slot, int k0) {
 #pragma unroll
     for (int i = 0; i < A_CHUNKS; ++i) {
       const int ch = tid + i * NT, row = ch / KCH, kc = (ch % KCH) * 8;
-      const int m = min(m0 + row, M - 1), k = min(k0 + kc, K - 8);
+      const int m = GROUPED ? gathered[i] : min(m0 + row, M - 1), k = min(k0 + kc, K - 8);
       ra[slot][i] = *(const bf16x8*)(A + (size_t)m * K + k);
     }
   };
@@ -1245,6 +1265,51 @@ static void launch_tile(int kind, const bf16_t* A, const bf16_t* W, const EpiArg
     else
       hipLaunchKernelGGL((gemm_bf16_pingpong<192, EPI>), grid, dim3(512), 0, stream, A, W, e, M, N, K);
   }
+}
+
+// Grouped products: `members` matrices [N, K] of equal shape lie one below the other in the packed
+// W (every member whole strips of 16 rows: N % 16 == 0); tile t of bm rows of the product belongs
+// to member tile_member[t] (-1: empty, its block leaves at once); row m reads row rows_index[m]
+// of x (null: row m).  out has M rows (a multiple of bm).  Epilogues: SWIGLU and F32.
+extern "C" int llmlab_linear_grouped(const void* x, const void* w, int epilogue, void* out, int M, int N, int K,
+                                     int ldo, int n_out, const int* tile_member, const int* rows_index, int bm,
+                                     hipStream_t stream) {
+  LLMLAB_REQUIRE(M >= 0 && N > 0 && K > 0 && K % 8 == 0 && N % 16 == 0, "linear_grouped: bad sizes M=%d N=%d K=%d", M,
+                 N, K);
+  LLMLAB_REQUIRE((bm == 64 || bm == 128) && M % bm == 0, "linear_grouped: %d rows in tiles of %d", M, bm);
+  LLMLAB_REQUIRE(epilogue == EPI_SWIGLU || epilogue == EPI_F32, "linear_grouped: epilogue %d", epilogue);
+  if (epilogue == EPI_SWIGLU)
+    LLMLAB_REQUIRE(N % 32 == 0 && n_out > 0 && 2 * ((n_out + 15) / 16 * 16) == N,
+                   "linear_grouped(swiglu): %d weight rows do not interleave %d outputs", N, n_out);
+  else
+    LLMLAB_REQUIRE(n_out <= N && n_out > N - 16, "linear_grouped: n_out %d, N %d", n_out, N);
+  LLMLAB_REQUIRE(ldo >= n_out && tile_member != nullptr, "linear_grouped: output stride or tile table");
+  if (M == 0) return 0;
+  EpiArgs e{out, nullptr, 0, ldo, n_out, 0, 0, nullptr, nullptr, nullptr, nullptr, nullptr, nullptr, 0, 0, 0, 0, 0, 0,
+            tile_member, rows_index, (size_t)(N / 16) * (size_t)((K + 31) / 32) * 512};
+  const bf16_t* A = (const bf16_t*)x;
+  const bf16_t* W = (const bf16_t*)w;
+  // (the columns past n_out of an F32 product are the zero rows that pad a member to whole strips)
+  const int cols = epilogue == EPI_SWIGLU ? N : n_out;
+  if (bm == 64) {
+    dim3 grid((cols + 63) / 64, M / 64, 1);
+    if (epilogue == EPI_SWIGLU)
+      hipLaunchKernelGGL((gemm_bf16_tiled<64, 64, 64, 2, 2, EPI_SWIGLU, true>), grid, dim3(256), 0, stream, A, W, e, M,
+                         cols, K);
+    else
+      hipLaunchKernelGGL((gemm_bf16_tiled<64, 64, 64, 2, 2, EPI_F32, true>), grid, dim3(256), 0, stream, A, W, e, M,
+                         cols, K);
+  } else {
+    dim3 grid((cols + 127) / 128, M / 128, 1);
+    if (epilogue == EPI_SWIGLU)
+      hipLaunchKernelGGL((gemm_bf16_tiled<128, 128, 64, 1, 4, EPI_SWIGLU, true>), grid, dim3(256), 0, stream, A, W, e,
+                         M, cols, K);
+    else
+      hipLaunchKernelGGL((gemm_bf16_tiled<128, 128, 64, 1, 4, EPI_F32, true>), grid, dim3(256), 0, stream, A, W, e, M,
+                         cols, K);
+  }
+  LLMLAB_LAUNCH_CHECK("linear_grouped");
+  return 0;
 }
 
 // Whether (and into how many pieces along K) a product that adds into float32 rows should

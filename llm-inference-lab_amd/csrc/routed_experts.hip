@@ -132,3 +132,110 @@ extern "C" int llmlab_moe_add_chosen(float* resid, const void* src, int src_dtyp
   LLMLAB_LAUNCH_CHECK("moe_add_chosen");
   return 0;
 }
+
+// ------------------------------------------------------------------ rows sorted by expert
+// The (row, choice) pairs of a step, sorted by expert into tiles of `bm` places that a grouped
+// product walks: every expert's pairs are consecutive and start at a multiple of bm.
+//   place_of[rows * top]   the place of a pair (-1: the pair chose no expert with tensors)
+//   place_row[capacity]    the row of x at a place (-1: the place is padding)
+//   tile_member[capacity / bm]   the expert of a tile of places (-1: past the last tile in use)
+// capacity = (pairs + experts * (bm - 1)) rounded up to whole tiles, whatever the choice: the
+// buffers and the grids that walk them have sizes the host knows.  One block: counts by atomic
+// adds in LDS, a scan over the experts, places handed out by atomic adds in LDS.  Which place
+// of its expert a pair gets depends on the order of those adds; no result does, because a row
+// of a product depends on that row alone.
+constexpr int PLAN_MAX_EXPERTS = 1024;
+
+__global__ __launch_bounds__(1024) void moe_plan_kernel(const int* __restrict__ chosen, int pairs, int experts, int bm,
+                                                        int capacity, int* __restrict__ place_of,
+                                                        int* __restrict__ place_row, int* __restrict__ tile_member,
+                                                        int top) {
+  __shared__ int s_count[PLAN_MAX_EXPERTS], s_start[PLAN_MAX_EXPERTS];
+  const int tid = threadIdx.x, nt = blockDim.x;
+  for (int e = tid; e < experts; e += nt) s_count[e] = 0;
+  for (int i = tid; i < capacity; i += nt) place_row[i] = -1;
+  for (int t = tid; t < capacity / bm; t += nt) tile_member[t] = -1;
+  __syncthreads();
+  for (int p = tid; p < pairs; p += nt) {
+    const int e = chosen[p];
+    if (e >= 0 && e < experts) atomicAdd(&s_count[e], 1);
+  }
+  __syncthreads();
+  if (tid == 0) {
+    int at = 0;
+    for (int e = 0; e < experts; ++e) {
+      s_start[e] = at;
+      at += (s_count[e] + bm - 1) / bm * bm;
+    }
+  }
+  __syncthreads();
+  for (int e = tid; e < experts; e += nt) {
+    const int first = s_start[e] / bm, tiles = (s_count[e] + bm - 1) / bm;
+    for (int t = 0; t < tiles; ++t) tile_member[first + t] = e;
+    s_count[e] = 0;                      // from here on: places handed out
+  }
+  __syncthreads();
+  for (int p = tid; p < pairs; p += nt) {
+    const int e = chosen[p];
+    int place = -1;
+    if (e >= 0 && e < experts) {
+      place = s_start[e] + atomicAdd(&s_count[e], 1);
+      place_row[place] = p / top;
+    }
+    place_of[p] = place;
+  }
+}
+
+extern "C" int llmlab_moe_plan(const int* chosen, int rows, int top, int experts, int bm, int capacity, int* place_of,
+                               int* place_row, int* tile_member, hipStream_t stream) {
+  LLMLAB_REQUIRE(rows >= 0 && top > 0 && experts > 0 && experts <= PLAN_MAX_EXPERTS && bm > 0,
+                 "moe_plan: bad sizes rows=%d top=%d experts=%d bm=%d", rows, top, experts, bm);
+  const long need = ((long)rows * top + (long)experts * (bm - 1) + bm - 1) / bm * bm;
+  LLMLAB_REQUIRE(capacity % bm == 0 && capacity >= need, "moe_plan: %d places for %d pairs of %d experts in tiles of %d",
+                 capacity, rows * top, experts, bm);
+  if (rows == 0) return 0;
+  hipLaunchKernelGGL(moe_plan_kernel, dim3(1), dim3(1024), 0, stream, chosen, rows * top, experts, bm, capacity, place_of,
+                     place_row, tile_member, top);
+  LLMLAB_LAUNCH_CHECK("moe_plan");
+  return 0;
+}
+
+// resid[r, :] += sum_k weights[r, k] * (y[place_of[r, k], :]  or, for a choice at or beyond
+// `experts` (an identity output), h[r, :]), the choices in their order.  One block a row.
+template <typename T>
+__global__ __launch_bounds__(256) void moe_combine_kernel(float* __restrict__ resid, const float* __restrict__ y,
+                                                          const T* __restrict__ h, const int* __restrict__ place_of,
+                                                          const int* __restrict__ chosen,
+                                                          const float* __restrict__ weights, int top, int experts,
+                                                          int hidden, const float* __restrict__ extra) {
+  const int row = blockIdx.x;
+  const int* places = place_of + (size_t)row * top;
+  const float* w = weights + (size_t)row * top;
+  for (int i = threadIdx.x; i < hidden; i += blockDim.x) {
+    float sum = 0.f;
+    for (int k = 0; k < top; ++k) {
+      const int place = places[k];
+      if (place >= 0)
+        sum += w[k] * y[(size_t)place * hidden + i];
+      else if (chosen[(size_t)row * top + k] >= experts)
+        sum += w[k] * to_float(h[(size_t)row * hidden + i]);
+    }
+    resid[(size_t)row * hidden + i] += sum;
+  }
+}
+
+extern "C" int llmlab_moe_combine(float* resid, const float* y, const void* h, int h_dtype, const int* place_of,
+                                  const int* chosen, const float* weights, int rows, int top, int experts, int hidden,
+                                  hipStream_t stream) {
+  LLMLAB_REQUIRE(rows >= 0 && top > 0 && hidden > 0, "moe_combine: bad sizes rows=%d top=%d hidden=%d", rows, top,
+                 hidden);
+  if (rows == 0) return 0;
+  if (h_dtype == DT_BF16)
+    hipLaunchKernelGGL(moe_combine_kernel<bf16_t>, dim3(rows), dim3(256), 0, stream, resid, y, (const bf16_t*)h, place_of,
+                       chosen, weights, top, experts, hidden, (const float*)nullptr);
+  else
+    hipLaunchKernelGGL(moe_combine_kernel<float>, dim3(rows), dim3(256), 0, stream, resid, y, (const float*)h, place_of,
+                       chosen, weights, top, experts, hidden, (const float*)nullptr);
+  LLMLAB_LAUNCH_CHECK("moe_combine");
+  return 0;
+}

@@ -79,6 +79,9 @@ class DispatchRules:
     # Debug only: a product that the tiled kernel cuts gets this many pieces whatever the
     # estimate says (0: the estimate decides).
     forced_tiled_pieces: int = 0
+    # Debug only: the experts of a mixture run one after the other over all rows with the plain
+    # products (what float32 does) instead of as grouped products over rows sorted by expert.
+    experts_one_by_one: bool = False
     # ``graph="auto"`` (engine/step.py): what one call into the kernel libraries costs the
     # host that makes it through ctypes, and the rate at which a decode step streams its
     # weights and its cache.  A decode step replayed from a HIP graph costs the host

@@ -86,6 +86,17 @@ class StackedWeight:
         return self.data.element_size()
 
 
+class MoePlan:
+    """The rows of a step sorted by expert (``HipOps.moe_plan``): ``capacity`` places in tiles of
+    ``bm``; ``place_of [rows, top]``, ``place_row [capacity]``, ``tile_member [capacity / bm]``."""
+
+    __slots__ = ("bm", "capacity", "place_of", "place_row", "tile_member")
+
+    def __init__(self, bm, capacity, place_of, place_row, tile_member):
+        self.bm, self.capacity = int(bm), int(capacity)
+        self.place_of, self.place_row, self.tile_member = place_of, place_row, tile_member
+
+
 class LaunchRecord:
     """The calls into the kernel libraries that a part made while it was recorded, so that
     the same part under the same conditions can make them again without its Python code:
@@ -240,6 +251,9 @@ class HipOps:
         c.llmlab_gate_heads.restype = _c_int
         c.llmlab_add_row_vector.argtypes = [_c_ptr, _c_ptr, _c_int, _c_int, _c_ptr]
         c.llmlab_add_row_vector.restype = _c_int
+        c.llmlab_linear_grouped.argtypes = [_c_ptr, _c_ptr, _c_int, _c_ptr, _c_int, _c_int, _c_int, _c_int, _c_int,
+                                            _c_ptr, _c_ptr, _c_int, _c_ptr]
+        c.llmlab_linear_grouped.restype = _c_int
         for fn in (c.llmlab_embed, c.llmlab_rmsnorm, c.llmlab_rope_kv_write, c.llmlab_rope_inplace,
                    c.llmlab_linear, c.llmlab_sample, c.llmlab_skinny_linear,
                    c.llmlab_linear_partials, c.llmlab_linear_qkv):
@@ -1067,6 +1081,12 @@ class HipOps:
                 lib.llmlab_moe_add_chosen.argtypes = [_c_ptr, _c_ptr, _c_int, _c_ptr, _c_ptr, _c_int, _c_int, _c_int,
                                                       _c_int, _c_int, _c_ptr]
                 lib.llmlab_moe_add_chosen.restype = _c_int
+                lib.llmlab_moe_plan.argtypes = [_c_ptr, _c_int, _c_int, _c_int, _c_int, _c_int, _c_ptr, _c_ptr, _c_ptr,
+                                                _c_ptr]
+                lib.llmlab_moe_plan.restype = _c_int
+                lib.llmlab_moe_combine.argtypes = [_c_ptr, _c_ptr, _c_ptr, _c_int, _c_ptr, _c_ptr, _c_ptr, _c_int, _c_int,
+                                                   _c_int, _c_int, _c_ptr]
+                lib.llmlab_moe_combine.restype = _c_int
             self._mixer_libs[kind] = lib
             self.loaded_libraries.append(lib._name)
         return lib
@@ -1098,8 +1118,72 @@ class HipOps:
         return stacked.data[e * stacked.n:(e + 1) * stacked.n]
 
     def moe_grouped(self, dtype) -> bool:
-        """Whether the experts of this dtype run as grouped products over rows sorted by expert."""
-        return False
+        """Whether the experts of this dtype run as grouped products over rows sorted by expert
+        (bfloat16: the tiled matrix-core kernel in its grouped form; float32 runs every expert over
+        all rows with the plain 32-bit products)."""
+        return dtype == torch.bfloat16 and not self.rules.experts_one_by_one
+
+    def moe_plan(self, chosen, num_experts: int, scratch) -> "MoePlan":
+        """Sort the ``(row, choice)`` pairs of ``chosen [rows, top]`` by expert into tiles of places
+        for the grouped products; choices at or beyond ``num_experts`` (outputs without tensors)
+        get no place.  ``scratch(name, shape, dtype)`` hands out the plan's buffers."""
+        lib = self._mixer_lib("routed_experts")
+        self._need(chosen, "chosen experts", torch.int32)
+        rows, top = chosen.shape
+        pairs = rows * top
+        # tiles of 128 places once an expert's share of the rows fills several of them
+        bm = 128 if pairs >= 512 * num_experts else 64
+        capacity = (pairs + num_experts * (bm - 1) + bm - 1) // bm * bm
+        plan = MoePlan(bm, capacity, scratch("experts.place_of", (rows, top), torch.int32),
+                       scratch("experts.place_row", (capacity,), torch.int32),
+                       scratch("experts.tile_member", (capacity // bm,), torch.int32))
+        self._call(lib.llmlab_moe_plan, self._ptr(chosen), rows, top, int(num_experts), bm, capacity,
+                   self._ptr(plan.place_of), self._ptr(plan.place_row), self._ptr(plan.tile_member), self._stream(),
+                   lib=lib)
+        return plan
+
+    def _grouped(self, x, stacked: "StackedWeight", plan: "MoePlan", out, epilogue, n_out, rows_index) -> None:
+        w = stacked.data
+        if not isinstance(w, PackedWeight) or x.dtype != torch.bfloat16:
+            raise TypeError("grouped products are bfloat16 products over a packed stack of matrices")
+        self._need(x, "grouped product input", torch.bfloat16)
+        self._need(out, "grouped product output")
+        if x.shape[1] != stacked.k or out.shape[0] != plan.capacity or out.shape[1] != n_out:
+            raise ValueError(f"grouped product: x {tuple(x.shape)}, members [{stacked.n}, {stacked.k}], "
+                             f"out {tuple(out.shape)}, {plan.capacity} places")
+        if rows_index is None and x.shape[0] != plan.capacity:
+            raise ValueError("grouped product: one row of x per place")
+        self._call(self._core.llmlab_linear_grouped, self._ptr(x), self._ptr(w), epilogue, self._ptr(out),
+                   plan.capacity, stacked.padded, stacked.k, out.stride(0), int(n_out), self._ptr(plan.tile_member),
+                   self._ptr(rows_index), plan.bm, self._stream())
+
+    def moe_gate_up(self, h, w_gate_up: "StackedWeight", plan: "MoePlan", act) -> None:
+        """``act[place] = silu(h[row] Wg_e^T) * (h[row] Wu_e^T)`` for every place of the plan, ``e`` the
+        expert of the place's tile and ``row`` the row of ``h`` at the place."""
+        if act.dtype != torch.bfloat16 or 2 * ((act.shape[1] + 15) // 16 * 16) != w_gate_up.n:
+            raise ValueError("moe_gate_up: the experts' gate and up rows do not interleave the outputs")
+        self._grouped(h, w_gate_up, plan, act, EPI_SWIGLU, act.shape[1], plan.place_row)
+
+    def moe_down(self, act, w_down: "StackedWeight", plan: "MoePlan", y) -> None:
+        """``y[place] = act[place] Wd_e^T`` in float32."""
+        if y.dtype != torch.float32 or y.shape[1] != w_down.n:
+            raise ValueError("moe_down: the output is float32 [places, hidden]")
+        self._grouped(act, w_down, plan, y, EPI_F32, w_down.n, None)
+
+    def moe_combine(self, resid, y, plan: "MoePlan", chosen, weights, num_experts: int, h) -> None:
+        """``resid[r] += sum_k weights[r, k] * y[place of (r, k)]``, the choices in their order; a
+        choice at or beyond ``num_experts`` stands for ``h[r]`` itself."""
+        lib = self._mixer_lib("routed_experts")
+        self._need(resid, "residual stream", torch.float32)
+        self._need(y, "expert outputs", torch.float32)
+        self._need(h, "expert input")
+        rows, hidden = resid.shape
+        if (y.shape[1] != hidden or tuple(h.shape) != (rows, hidden) or chosen.shape[0] != rows
+                or tuple(weights.shape) != tuple(chosen.shape) or tuple(plan.place_of.shape) != tuple(chosen.shape)):
+            raise ValueError("moe_combine: shapes do not fit")
+        self._call(lib.llmlab_moe_combine, self._ptr(resid), self._ptr(y), self._ptr(h), _dt(h),
+                   self._ptr(plan.place_of), self._ptr(chosen), self._ptr(weights), rows, chosen.shape[1],
+                   int(num_experts), hidden, self._stream(), lib=lib)
 
     def moe_select(self, logits, correction, groups: int, groups_keep: int, scale: float, chosen, weights) -> None:
         """Per row of the router's float32 ``logits [rows, outputs]``: scores ``softmax(logits)``; choice

@@ -80,13 +80,11 @@ class GQAAttention(Mixer):
     def tensor_specs(self):
         t, h = self.tensor_names, self.hidden_size
         q_size, kv_size = self.num_heads * self.file_head_dim, self.num_kv_heads * self.file_head_dim
-        specs = {
-            t["q_weight"]: TensorSpec((q_size, h), MATRIX),
-            t["k_weight"]: TensorSpec((kv_size, h), MATRIX),
-            t["o_weight"]: TensorSpec((h, q_size), MATRIX),
-        }
+        # (the random-weights mode draws a tensor by its place in this list: the order stays)
+        specs = {t["q_weight"]: TensorSpec((q_size, h), MATRIX), t["k_weight"]: TensorSpec((kv_size, h), MATRIX)}
         if not self.values_from_keys:
             specs[t["v_weight"]] = TensorSpec((kv_size, h), MATRIX)
+        specs[t["o_weight"]] = TensorSpec((h, q_size), MATRIX)
         if self.output_gate:
             specs[t["gate_weight"]] = TensorSpec((self.num_heads, h), MATRIX)
         if self.qkv_bias:

@@ -115,7 +115,9 @@ class RoutedExperts(FeedForward):
                 ops.linear_swiglu(h, ops.stacked_member(self.w_gate_up, e), act)
                 ops.linear_logits(act, ops.stacked_member(self.w_down, e), y)
                 ops.moe_add_chosen(residual, y, chosen, weights, e, e + 1)
-        if self.identity:
+            if self.identity:
+                ops.moe_add_chosen(residual, h, chosen, weights, self.num_experts, self.outputs)
+        elif self.identity:
             ops.moe_add_chosen(residual, h, chosen, weights, self.num_experts, self.outputs)
         if self.shared is not None:
             self.shared.forward(h, residual, ctx)
@@ -127,7 +129,7 @@ class RoutedExperts(FeedForward):
         ops.moe_gate_up(h, self.w_gate_up, plan, act)
         y = ctx.scratch("experts.out", (plan.capacity, self.hidden_size), torch.float32)
         ops.moe_down(act, self.w_down, plan, y)
-        ops.moe_combine(residual, y, plan, chosen, weights, self.num_experts)
+        ops.moe_combine(residual, y, plan, chosen, weights, self.num_experts, h)     # (identity outputs too)
 
     @property
     def graph_safe(self):

@@ -218,9 +218,15 @@ def test_the_mixture_of_experts_alone(backend, dtype, rows, shape):
     resid = randn(rows, width, seed=12)
     got = resid.clone().to(ops.device)
     part.forward(h.to(dtype).to(ops.device), got, Scratch(ops.device))
-    if getattr(ops, "synchronize", None):
-        ops.synchronize()
     close(got.cpu()[sure], (resid.to(F64) + want)[sure], dtype, "stream + mixture", f32=5e-5, bf16=4e-2)
+    if backend == "hip" and dtype == torch.bfloat16:
+        # the same with the experts one after the other over all rows (what float32 does) instead
+        # of grouped products over rows sorted by expert
+        assert ops.moe_grouped(dtype)
+        with ops.debug.force(experts_one_by_one=True):
+            again = resid.clone().to(ops.device)
+            part.forward(h.to(dtype).to(ops.device), again, Scratch(ops.device))
+        close(again.cpu()[sure], (resid.to(F64) + want)[sure], dtype, "stream + mixture, expert by expert", bf16=4e-2)
 
 
 # ------------------------------------------------------------------ window edges, far keys
