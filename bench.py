@@ -3,7 +3,7 @@
     python bench.py [--gpus 1] [--steps K] [--warmup W] [--batch B] [--context S]
                     [--shape 0.5b|7b|32b] [--layers L] [--dtype bf16|f32]
     python bench.py --mixed [--shape 7b] [--requests 64] [--chunk 512] [--outputs 64]
-    python bench.py --design vivevik [--size small|medium|large] [--context 2048]
+    python bench.py --design vivevik|ruvalorn [--size small|medium|large] [--context 2048]
 
 Default: the layer sizes of the Qwen2.5-0.5B shape with seeded random weights,
 batch 8, context 4096, bfloat16.  A "step" is one decode step of the whole
@@ -42,6 +42,8 @@ timed steps, so that the profile holds those and not the filling of the caches
 attention layers beside windowed attention layers with a sink, some of which read an earlier
 layer's keys and values) at layer sizes of real models, beside the Qwen2 decoder with the same
 width, heads, feed-forward width and number of layers; one JSON line, a record per size.
+``--design ruvalorn``: the same for the Ruvalorn design (windowed attention whose values are its
+keys, a gate per head, mixtures of experts behind a grouped router, some layers run twice).
 
 ``--mixed``: many requests with prompts of different lengths go through the
 scheduler with a small token budget, so that portions of prompts run beside the
@@ -147,6 +149,52 @@ def vivevik_flops(cfg, tokens):
     return total + 2 * w * cfg.vocab
 
 
+# ``--design ruvalorn``: per size (experts, expert width, chosen per token, identity outputs, shared
+# expert's width): chosen * expert width + shared width is the dense feed-forward's width, so a
+# token does the Qwen2 decoder's arithmetic.  The first layer's feed-forward is dense, the others
+# are mixtures; layers 1 .. n-2 run twice (so that the layer RUNS equal the Qwen2 decoder's
+# layers), windows of 1,024 positions, half of every head rotates.
+RUVALORN_EXPERTS = {"small": (32, 512, 8, 4, 768), "medium": (32, 1024, 8, 4, 2816), "large": (32, 2048, 8, 4, 2560)}
+
+
+def ruvalorn_config(size):
+    import llm_inference_lab_amd as lab
+    width, heads, kv, dim, ff, runs = DESIGN_SIZES[size]
+    experts, expert_ff, top, identity, shared = RUVALORN_EXPERTS[size]
+    layers = runs // 2 + 1                       # 1 + 2 * (layers - 2) + 1 runs
+    listed = []
+    for i in range(layers):
+        mixer = dict(heads=heads, kv_heads=kv, dim=dim, vdim=dim, scale=dim ** -0.5, mask=dict(size=DESIGN_WINDOW),
+                     rot=dict(dims=dim // 2, base=1e6))
+        mlp = dict(kind="dense", ff=ff) if i == 0 else dict(
+            kind="moe", expert=dict(ff=expert_ff), shared=dict(ff=shared),
+            router=dict(experts=experts, identity=identity, top=top, scale=2.5, groups=dict(count=4, keep=3)))
+        listed.append(dict(type="attention", mixer=mixer, mlp=mlp))
+    return lab.RuvalornConfig.from_dict(dict(architecture="Ruvalorn", vocab=DESIGN_VOCAB, width=width,
+                                             norm=dict(eps=1e-6), layers=listed,
+                                             loop=dict(start=1, stop=layers - 1, times=2)))
+
+
+def ruvalorn_flops(cfg, tokens):
+    """Multiply-adds times two of one prompt of ``tokens`` positions, as the design defines them
+    (one key projection; a chosen identity output costs nothing: the share of the router's
+    outputs that are experts is taken as the share of the choices)."""
+    w, total = cfg.width, 0
+    for i, _ in cfg.runs():
+        l = cfg.layers[i]
+        q, k = l.heads * l.dim, l.kv_heads * l.dim
+        total += tokens * 2 * (w * (q + k + l.heads) + q * w)
+        total += 4 * sum(min(p + 1, l.window or tokens) for p in range(tokens)) * l.heads * l.dim
+        f = l.mlp
+        if f is not None and f.kind == "dense":
+            total += tokens * 6 * w * f.ff
+        elif f is not None:
+            r = f.router
+            total += tokens * (2 * w * (r.experts + r.identity) + 6 * w * (f.shared_ff or 0)
+                               + 6 * w * f.ff * r.top * r.experts / (r.experts + r.identity))
+    return total + 2 * w * cfg.vocab
+
+
 def design_run(args, bracket=None):
     """``--design vivevik``: both models at each size, one after the other on the same GPU.
     ``--only-model``, ``--only-prefill`` / ``--only-decode`` and ``--batch`` narrow the run (for
@@ -166,7 +214,8 @@ def design_run(args, bracket=None):
                                               num_key_value_heads=kv, head_dim=dim, tie_word_embeddings=True))
         record[size] = {"width": width, "heads": heads, "kv_heads": kv, "head_dim": dim, "ff": ff, "layers": layers,
                         "context": context, "window": DESIGN_WINDOW}
-        for label, cfg in (("vivevik", vivevik_config(size)), ("qwen2", qwen)):
+        design = ruvalorn_config(size) if args.design == "ruvalorn" else vivevik_config(size)
+        for label, cfg in ((args.design, design), ("qwen2", qwen)):
             if args.only_model and label != args.only_model:
                 continue
             expected = CausalLM(get_architecture(cfg.architecture).build_spec(cfg)).tensor_specs()
@@ -179,7 +228,9 @@ def design_run(args, bracket=None):
                                 graph=False if args.no_graph else args.graph)
             view = types.SimpleNamespace(vocab_size=engine.spec.vocab_size)
             runs = Runs(engine, view, context, args.dtype, args.samples, bracket)
-            flops = vivevik_flops(cfg, args.prefill_tokens) if label == "vivevik" else prefill_flops(cfg, args.prefill_tokens)
+            flops = (vivevik_flops(cfg, args.prefill_tokens) if label == "vivevik" else
+                     ruvalorn_flops(cfg, args.prefill_tokens) if label == "ruvalorn" else
+                     prefill_flops(cfg, args.prefill_tokens))
             out = {"weight_bytes_per_step": engine.weight_bytes_per_step()}
             if not args.only_decode:
                 out["prefill"] = runs.prefill(args.prefill_tokens, flops=flops)
@@ -199,7 +250,7 @@ def design_run(args, bracket=None):
             del engine, runs
             torch.cuda.empty_cache()
         print(f"[bench] {size}: {json.dumps(record[size])}", file=sys.stderr, flush=True)
-    print(json.dumps({"metric": "design_throughput", "design": "vivevik", "beside": "qwen2", "dtype": args.dtype,
+    print(json.dumps({"metric": "design_throughput", "design": args.design, "beside": "qwen2", "dtype": args.dtype,
                       "data": "synthetic", "unit": "tokens/s", "prefill_tokens": args.prefill_tokens,
                       "sizes": record}))
 
@@ -710,10 +761,10 @@ def main():
                     help="fix a choice of the kernels for the whole run, to compare variants: a keyword of "
                          "engine.ops.debug.force, values separated by ':' (attention_splits=64:8, "
                          "attention_merge_kernel=64, gemm_tile=129)")
-    ap.add_argument("--design", choices=["vivevik"], default=None,
+    ap.add_argument("--design", choices=["vivevik", "ruvalorn"], default=None,
                     help="throughput of another design beside the Qwen2 decoder of equal size")
     ap.add_argument("--size", choices=sorted(DESIGN_SIZES), default=None, help="--design: one size only")
-    ap.add_argument("--only-model", choices=["vivevik", "qwen2"], default=None, help="--design: one of the two models only")
+    ap.add_argument("--only-model", choices=["vivevik", "ruvalorn", "qwen2"], default=None, help="--design: one of the two models only")
     ap.add_argument("--only-decode", action="store_true", help="--design: decode at --batch only, no prefill")
     ap.add_argument("--side", choices=["7b", "32b", "f32", "peaks"], help=argparse.SUPPRESS)
     args = ap.parse_args()

@@ -1273,10 +1273,12 @@ static void launch_tile(int kind, const bf16_t* A, const bf16_t* W, const EpiArg
 // of x (null: row m).  out has M rows (a multiple of bm).  Epilogues: SWIGLU and F32.
 extern "C" int llmlab_linear_grouped(const void* x, const void* w, int epilogue, void* out, int M, int N, int K,
                                      int ldo, int n_out, const int* tile_member, const int* rows_index, int bm,
-                                     hipStream_t stream) {
+                                     int wide, hipStream_t stream) {
   LLMLAB_REQUIRE(M >= 0 && N > 0 && K > 0 && K % 8 == 0 && N % 16 == 0, "linear_grouped: bad sizes M=%d N=%d K=%d", M,
                  N, K);
   LLMLAB_REQUIRE((bm == 64 || bm == 128) && M % bm == 0, "linear_grouped: %d rows in tiles of %d", M, bm);
+  if (g_force_tile == 129) wide = 0;
+  if (g_force_tile == 131) wide = 1;
   LLMLAB_REQUIRE(epilogue == EPI_SWIGLU || epilogue == EPI_F32, "linear_grouped: epilogue %d", epilogue);
   if (epilogue == EPI_SWIGLU)
     LLMLAB_REQUIRE(N % 32 == 0 && n_out > 0 && 2 * ((n_out + 15) / 16 * 16) == N,
@@ -1298,6 +1300,15 @@ extern "C" int llmlab_linear_grouped(const void* x, const void* w, int epilogue,
                          cols, K);
     else
       hipLaunchKernelGGL((gemm_bf16_tiled<64, 64, 64, 2, 2, EPI_F32, true>), grid, dim3(256), 0, stream, A, W, e, M,
+                         cols, K);
+  } else if (wide) {
+    // (tiles of 128 rows and 256 columns, eight waves side by side)
+    dim3 grid((cols + 255) / 256, M / 128, 1);
+    if (epilogue == EPI_SWIGLU)
+      hipLaunchKernelGGL((gemm_bf16_tiled<128, 256, 64, 1, 8, EPI_SWIGLU, true>), grid, dim3(512), 0, stream, A, W, e,
+                         M, cols, K);
+    else
+      hipLaunchKernelGGL((gemm_bf16_tiled<128, 256, 64, 1, 8, EPI_F32, true>), grid, dim3(512), 0, stream, A, W, e, M,
                          cols, K);
   } else {
     dim3 grid((cols + 127) / 128, M / 128, 1);

@@ -84,6 +84,54 @@ __global__ __launch_bounds__(64) void moe_select_kernel(const float* __restrict_
   }
 }
 
+// The same for a router of up to 64 outputs: a lane an output, everything in registers, no LDS
+// and no barrier (the values cross lanes by shuffles).
+__global__ __launch_bounds__(64) void moe_select_wave_kernel(const float* __restrict__ logits,
+                                                             const float* __restrict__ correction, int outputs, int groups,
+                                                             int keep, int top, float scale, int* __restrict__ chosen,
+                                                             float* __restrict__ weights) {
+  const int row = blockIdx.x, lane = threadIdx.x;
+  const bool mine = lane < outputs;
+  const float z = mine ? logits[(size_t)row * outputs + lane] : -INFINITY;
+  float m = z;
+  for (int o = 32; o > 0; o >>= 1) m = fmaxf(m, __shfl_xor(m, o));
+  const float p = mine ? expf(z - m) : 0.f;
+  float sum = p;
+  for (int o = 32; o > 0; o >>= 1) sum += __shfl_xor(sum, o);
+  const float score = p * (1.f / sum);
+  float choice = mine ? score + correction[lane] : -INFINITY;
+  if (keep < groups) {
+    const int per = outputs / groups, g = mine ? lane / per : 0;
+    float best = -INFINITY;
+    for (int i = 0; i < per; ++i) best = fmaxf(best, __shfl(choice, g * per + i));
+    int before = 0;
+    for (int o = 0; o < groups; ++o) {
+      const float other = __shfl(best, o * per);
+      before += (other > best) || (other == best && o < g);
+    }
+    if (before >= keep) choice = -INFINITY;
+  }
+  for (int k = 0; k < top; ++k) {
+    float best = choice;
+    int at = mine ? lane : outputs;
+    for (int o = 32; o > 0; o >>= 1) {
+      const float ob = __shfl_xor(best, o);
+      const int oa = __shfl_xor(at, o);
+      if (ob > best || (ob == best && oa < at)) {
+        best = ob;
+        at = oa;
+      }
+    }
+    at = min(at, outputs - 1);
+    const float s_at = __shfl(score, at);
+    if (lane == 0) {
+      chosen[(size_t)row * top + k] = at;
+      weights[(size_t)row * top + k] = s_at * scale;
+    }
+    if (lane == at) choice = -INFINITY;      // taken
+  }
+}
+
 extern "C" int llmlab_moe_select(const float* logits, const float* correction, int rows, int outputs, int groups,
                                  int keep, int top, float scale, int* chosen, float* weights, hipStream_t stream) {
   LLMLAB_REQUIRE(rows >= 0 && outputs > 0 && outputs <= SELECT_MAX_OUTPUTS,
@@ -92,8 +140,12 @@ extern "C" int llmlab_moe_select(const float* logits, const float* correction, i
                      top <= keep * (outputs / groups),
                  "moe_select: %d outputs in %d groups of which %d are kept, top %d", outputs, groups, keep, top);
   if (rows == 0) return 0;
-  hipLaunchKernelGGL(moe_select_kernel, dim3(rows), dim3(64), 0, stream, logits, correction, outputs, groups, keep,
-                     top, scale, chosen, weights);
+  if (outputs <= WAVE)
+    hipLaunchKernelGGL(moe_select_wave_kernel, dim3(rows), dim3(64), 0, stream, logits, correction, outputs, groups,
+                       keep, top, scale, chosen, weights);
+  else
+    hipLaunchKernelGGL(moe_select_kernel, dim3(rows), dim3(64), 0, stream, logits, correction, outputs, groups, keep,
+                       top, scale, chosen, weights);
   LLMLAB_LAUNCH_CHECK("moe_select");
   return 0;
 }
@@ -211,7 +263,7 @@ __global__ __launch_bounds__(256) void moe_combine_kernel(float* __restrict__ re
   const int row = blockIdx.x;
   const int* places = place_of + (size_t)row * top;
   const float* w = weights + (size_t)row * top;
-  for (int i = threadIdx.x; i < hidden; i += blockDim.x) {
+  for (int i = blockIdx.y * blockDim.x + threadIdx.x; i < hidden; i += gridDim.y * blockDim.x) {
     float sum = 0.f;
     for (int k = 0; k < top; ++k) {
       const int place = places[k];
@@ -230,11 +282,14 @@ extern "C" int llmlab_moe_combine(float* resid, const float* y, const void* h, i
   LLMLAB_REQUIRE(rows >= 0 && top > 0 && hidden > 0, "moe_combine: bad sizes rows=%d top=%d hidden=%d", rows, top,
                  hidden);
   if (rows == 0) return 0;
+  // few rows: the columns of a row are spread over several blocks, so that the chip has work
+  const int across = rows >= 1024 ? 1 : min((hidden + 255) / 256, max(1, 1024 / rows));
+  const dim3 grid(rows, across);
   if (h_dtype == DT_BF16)
-    hipLaunchKernelGGL(moe_combine_kernel<bf16_t>, dim3(rows), dim3(256), 0, stream, resid, y, (const bf16_t*)h, place_of,
+    hipLaunchKernelGGL(moe_combine_kernel<bf16_t>, grid, dim3(256), 0, stream, resid, y, (const bf16_t*)h, place_of,
                        chosen, weights, top, experts, hidden, (const float*)nullptr);
   else
-    hipLaunchKernelGGL(moe_combine_kernel<float>, dim3(rows), dim3(256), 0, stream, resid, y, (const float*)h, place_of,
+    hipLaunchKernelGGL(moe_combine_kernel<float>, grid, dim3(256), 0, stream, resid, y, (const float*)h, place_of,
                        chosen, weights, top, experts, hidden, (const float*)nullptr);
   LLMLAB_LAUNCH_CHECK("moe_combine");
   return 0;

@@ -82,6 +82,9 @@ class DispatchRules:
     # Debug only: the experts of a mixture run one after the other over all rows with the plain
     # products (what float32 does) instead of as grouped products over rows sorted by expert.
     experts_one_by_one: bool = False
+    # Grouped products in tiles of 128 rows: from this many columns of a member on the tile is
+    # 256 columns wide (eight waves) instead of 128.
+    grouped_wide_min_columns: int = 1024
     # ``graph="auto"`` (engine/step.py): what one call into the kernel libraries costs the
     # host that makes it through ctypes, and the rate at which a decode step streams its
     # weights and its cache.  A decode step replayed from a HIP graph costs the host

@@ -252,7 +252,7 @@ class HipOps:
         c.llmlab_add_row_vector.argtypes = [_c_ptr, _c_ptr, _c_int, _c_int, _c_ptr]
         c.llmlab_add_row_vector.restype = _c_int
         c.llmlab_linear_grouped.argtypes = [_c_ptr, _c_ptr, _c_int, _c_ptr, _c_int, _c_int, _c_int, _c_int, _c_int,
-                                            _c_ptr, _c_ptr, _c_int, _c_ptr]
+                                            _c_ptr, _c_ptr, _c_int, _c_int, _c_ptr]
         c.llmlab_linear_grouped.restype = _c_int
         for fn in (c.llmlab_embed, c.llmlab_rmsnorm, c.llmlab_rope_kv_write, c.llmlab_rope_inplace,
                    c.llmlab_linear, c.llmlab_sample, c.llmlab_skinny_linear,
@@ -1155,7 +1155,9 @@ class HipOps:
             raise ValueError("grouped product: one row of x per place")
         self._call(self._core.llmlab_linear_grouped, self._ptr(x), self._ptr(w), epilogue, self._ptr(out),
                    plan.capacity, stacked.padded, stacked.k, out.stride(0), int(n_out), self._ptr(plan.tile_member),
-                   self._ptr(rows_index), plan.bm, self._stream())
+                   self._ptr(rows_index), plan.bm,
+                   1 if plan.bm == 128 and stacked.padded >= self.rules.grouped_wide_min_columns else 0,
+                   self._stream())
 
     def moe_gate_up(self, h, w_gate_up: "StackedWeight", plan: "MoePlan", act) -> None:
         """``act[place] = silu(h[row] Wg_e^T) * (h[row] Wu_e^T)`` for every place of the plan, ``e`` the
