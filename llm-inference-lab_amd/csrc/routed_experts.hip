@@ -85,7 +85,13 @@ __global__ __launch_bounds__(64) void moe_select_kernel(const float* __restrict_
 }
 
 // The same for a router of up to 64 outputs: a lane an output, everything in registers, no LDS
-// and no barrier (the values cross lanes by shuffles).
+// and no barrier.  A lane finds its place in the order (value down, index up) by reading every
+// other lane's value in turn (a read of a lane that is the same for the whole wave, which costs a
+// few clocks; a chain of lane-to-lane exchanges per chosen output would cost a hundred each).
+__device__ __forceinline__ float lane_value(float v, int lane) {
+  return __builtin_bit_cast(float, __builtin_amdgcn_readlane(__builtin_bit_cast(int, v), lane));
+}
+
 __global__ __launch_bounds__(64) void moe_select_wave_kernel(const float* __restrict__ logits,
                                                              const float* __restrict__ correction, int outputs, int groups,
                                                              int keep, int top, float scale, int* __restrict__ chosen,
@@ -93,42 +99,35 @@ __global__ __launch_bounds__(64) void moe_select_wave_kernel(const float* __rest
   const int row = blockIdx.x, lane = threadIdx.x;
   const bool mine = lane < outputs;
   const float z = mine ? logits[(size_t)row * outputs + lane] : -INFINITY;
-  float m = z;
-  for (int o = 32; o > 0; o >>= 1) m = fmaxf(m, __shfl_xor(m, o));
+  float m = -INFINITY;
+  for (int j = 0; j < outputs; ++j) m = fmaxf(m, lane_value(z, j));
   const float p = mine ? expf(z - m) : 0.f;
-  float sum = p;
-  for (int o = 32; o > 0; o >>= 1) sum += __shfl_xor(sum, o);
+  float sum = 0.f;
+  for (int j = 0; j < outputs; ++j) sum += lane_value(p, j);         // (in the order of the outputs, on every lane)
   const float score = p * (1.f / sum);
   float choice = mine ? score + correction[lane] : -INFINITY;
   if (keep < groups) {
-    const int per = outputs / groups, g = mine ? lane / per : 0;
-    float best = -INFINITY;
-    for (int i = 0; i < per; ++i) best = fmaxf(best, __shfl(choice, g * per + i));
-    int before = 0;
+    const int per = outputs / groups, g = mine ? lane / per : groups;
+    float best = -INFINITY;                    // of this lane's group
+    for (int j = 0; j < outputs; ++j) {
+      const float c = lane_value(choice, j);
+      if (j / per == g) best = fmaxf(best, c);
+    }
+    int before = 0;                            // groups that come before this lane's
     for (int o = 0; o < groups; ++o) {
-      const float other = __shfl(best, o * per);
+      const float other = lane_value(best, o * per);
       before += (other > best) || (other == best && o < g);
     }
     if (before >= keep) choice = -INFINITY;
   }
-  for (int k = 0; k < top; ++k) {
-    float best = choice;
-    int at = mine ? lane : outputs;
-    for (int o = 32; o > 0; o >>= 1) {
-      const float ob = __shfl_xor(best, o);
-      const int oa = __shfl_xor(at, o);
-      if (ob > best || (ob == best && oa < at)) {
-        best = ob;
-        at = oa;
-      }
-    }
-    at = min(at, outputs - 1);
-    const float s_at = __shfl(score, at);
-    if (lane == 0) {
-      chosen[(size_t)row * top + k] = at;
-      weights[(size_t)row * top + k] = s_at * scale;
-    }
-    if (lane == at) choice = -INFINITY;      // taken
+  int place = 0;                               // outputs that come before this lane's
+  for (int j = 0; j < outputs; ++j) {
+    const float c = lane_value(choice, j);
+    place += (c > choice) || (c == choice && j < lane);
+  }
+  if (mine && place < top) {
+    chosen[(size_t)row * top + place] = lane;
+    weights[(size_t)row * top + place] = score * scale;
   }
 }
 

@@ -8,7 +8,7 @@ import torch
 from ..config.spec import PartSpec
 from ..weights.loader import TensorSpec, MATRIX, VECTOR, INIT_ZEROS
 from .base import FeedForward, NormedInput
-from .feed_forward import interleave_gate_up
+from .feed_forward import interleave_gate_up, pad_columns
 from .registry import register_part, build_part
 
 
@@ -41,6 +41,7 @@ class RoutedExperts(FeedForward):
                  correction: bool = True, shared: Optional[PartSpec] = None):
         super().__init__(tensors)
         self.hidden_size, self.expert_size = int(hidden_size), int(expert_size)
+        self.kernel_size = (self.expert_size + 7) // 8 * 8       # (as in ``SwiGLU``: zeros behind an odd width)
         self.num_experts, self.identity, self.top = int(num_experts), int(identity), int(top)
         self.outputs = self.num_experts + self.identity
         self.scale, self.groups, self.groups_keep = float(scale), int(groups), int(groups_keep)
@@ -76,7 +77,6 @@ class RoutedExperts(FeedForward):
     def bind(self, tensors, ops, dtype):
         super().bind(tensors, ops, dtype)
         ops.check_product_sizes(self.hidden_size, dtype, "experts (hidden size)")
-        ops.check_product_sizes(self.expert_size, dtype, "experts (expert size)")
         t = self.tensor_names
         self.w_router = ops.prepare_weight(tensors[t["router"]].contiguous())
         self.correction = (tensors[t["correction"]].float().contiguous() if self.has_correction
@@ -89,7 +89,7 @@ class RoutedExperts(FeedForward):
             self.gate_up_rows = gate_up[0].shape[0]
             self.w_gate_up = ops.prepare_stacked(torch.cat(gate_up, dim=0).contiguous(), self.num_experts)
             del gate_up
-            self.w_down = ops.prepare_stacked(torch.cat([tensors[d] for _, _, d in names], dim=0).contiguous(),
+            self.w_down = ops.prepare_stacked(torch.cat([pad_columns(tensors[d], self.kernel_size) for _, _, d in names], dim=0).contiguous(),
                                               self.num_experts)
         if self.shared is not None:
             self.shared.bind(tensors, ops, dtype)
@@ -109,7 +109,7 @@ class RoutedExperts(FeedForward):
         if self.num_experts and getattr(ops, "moe_grouped", None) is not None and ops.moe_grouped(self.dtype):
             self._grouped(h, residual, ctx, chosen, weights)
         elif self.num_experts:
-            act = ctx.scratch("experts.act", (rows, self.expert_size), self.dtype)
+            act = ctx.scratch("experts.act", (rows, self.kernel_size), self.dtype)
             y = ctx.scratch("experts.out", (rows, self.hidden_size), torch.float32)
             for e in range(self.num_experts):
                 ops.linear_swiglu(h, ops.stacked_member(self.w_gate_up, e), act)
@@ -125,7 +125,7 @@ class RoutedExperts(FeedForward):
     def _grouped(self, h, residual, ctx, chosen, weights):
         ops, rows, top = self.ops, h.shape[0], self.top
         plan = ops.moe_plan(chosen, self.num_experts, ctx.scratch)
-        act = ctx.scratch("experts.act", (plan.capacity, self.expert_size), self.dtype)
+        act = ctx.scratch("experts.act", (plan.capacity, self.kernel_size), self.dtype)
         ops.moe_gate_up(h, self.w_gate_up, plan, act)
         y = ctx.scratch("experts.out", (plan.capacity, self.hidden_size), torch.float32)
         ops.moe_down(act, self.w_down, plan, y)

@@ -31,6 +31,15 @@ def interleave_gate_up(gate: torch.Tensor, up: torch.Tensor) -> torch.Tensor:
     return out
 
 
+def pad_columns(w: torch.Tensor, columns: int) -> torch.Tensor:
+    """``w [n, k]`` with zero columns behind it up to ``columns``."""
+    if w.shape[1] == columns:
+        return w.contiguous()
+    out = torch.zeros((w.shape[0], columns), dtype=w.dtype, device=w.device)
+    out[:, :w.shape[1]] = w
+    return out
+
+
 class SwiGLU(FeedForward):
     """``residual += (silu(h Wg^T) * (h Wu^T)) Wd^T`` with ``silu(z) = z / (1 +
     exp(-z))``; accumulators, the sigmoid and the product in float32.
@@ -45,6 +54,9 @@ class SwiGLU(FeedForward):
             raise ValueError(f"SwiGLU supports activation 'silu', got '{activation}'")
         self.hidden_size = int(hidden_size)
         self.intermediate_size = int(intermediate_size)
+        # the kernels' inner sizes are multiples of 8: an intermediate size that is not is laid out
+        # with zero rows of gate and up (whose activation is 0) and zero columns of down behind it
+        self.kernel_size = (self.intermediate_size + 7) // 8 * 8
         self.w_gate_up = self.w_down = None
 
     def tensor_specs(self):
@@ -58,18 +70,17 @@ class SwiGLU(FeedForward):
     def bind(self, tensors, ops, dtype):
         super().bind(tensors, ops, dtype)
         ops.check_product_sizes(self.hidden_size, dtype, "feed-forward (hidden size)")
-        ops.check_product_sizes(self.intermediate_size, dtype, "feed-forward (intermediate size)")
         t = self.tensor_names
         self.w_gate_up = ops.prepare_weight(
             interleave_gate_up(tensors[t["gate_weight"]], tensors[t["up_weight"]]))
-        self.w_down = ops.prepare_weight(tensors[t["down_weight"]].contiguous())
+        self.w_down = ops.prepare_weight(pad_columns(tensors[t["down_weight"]], self.kernel_size))
 
     takes_normed_input = True
     keeps_launches = True
 
     def forward(self, h, residual, ctx):
         rows = h.shape[0]
-        act = ctx.scratch("swiglu.act", (rows, self.intermediate_size), self.dtype)
+        act = ctx.scratch("swiglu.act", (rows, self.kernel_size), self.dtype)
         fuse = isinstance(h, NormedInput) and self.ops.can_fuse(rows, self.dtype, self.hidden_size,
                                                                  self.w_gate_up.shape[0])
         rms = h.rms() if fuse else None      # (folds pieces still owed to the stream; else the norm does)
@@ -79,7 +90,7 @@ class SwiGLU(FeedForward):
             if isinstance(h, NormedInput):
                 h = h.tensor()
             self.ops.linear_swiglu(h, self.w_gate_up, act)
-        splits = self.ops.split_count(rows, self.dtype, self.hidden_size, self.intermediate_size)
+        splits = self.ops.split_count(rows, self.dtype, self.hidden_size, self.kernel_size)
         if splits > 1 and hasattr(ctx, "pending") and ctx.pending is None:
             # a narrow output: the product is cut along the inner size so that it spreads
             # over the chip, and its pieces are left for the next reader of the stream

@@ -1,7 +1,7 @@
 """Ruvalorn configurations drawn at random (widths, head counts and sizes also beside the
 multiples of 16, how much of a head rotates, windows shorter and longer than the sequences and the
 16-token pages or none, dense feed-forwards, mixtures with and without groups, identity outputs
-and a shared expert, layers without a feed-forward, loops anywhere in the stack): mixed batches
+and a shared expert, feed-forward widths beside the multiples of 8, layers without a feed-forward, loops anywhere in the stack): mixed batches
 through the engine against the plain implementation, float32 tight and bfloat16 by the root mean
 square."""
 import random
@@ -21,16 +21,16 @@ def draw_mlp(rng):
     if kind == "none":
         return None
     if kind == "dense":
-        return R.dense(8 * rng.randint(2, 20))
+        return R.dense(rng.choice([8 * rng.randint(2, 20), 20, 36, 100]))
     per, count = rng.choice([1, 2, 3, 5]), rng.choice([1, 2, 4])
     outputs = per * count
     identity = rng.choice([0, 0, 1, per]) if outputs > 1 else 0
     identity = min(identity, outputs - 1)
     keep = rng.randint(1, count)
     top = rng.randint(1, min(keep * per, 4))
-    return R.moe(8 * rng.randint(1, 6), outputs - identity, top, identity=identity, scale=rng.choice([0.5, 1.0, 2.5]),
+    return R.moe(rng.choice([8 * rng.randint(1, 6), 12, 20]), outputs - identity, top, identity=identity, scale=rng.choice([0.5, 1.0, 2.5]),
                  groups=None if count == 1 and rng.random() < 0.5 else (count, keep),
-                 shared=rng.choice([None, 8 * rng.randint(1, 8)]))
+                 shared=rng.choice([None, 8 * rng.randint(1, 8), 28]))
 
 
 def draw_config(seed):
