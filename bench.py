@@ -227,6 +227,7 @@ def design_run(args, bracket=None):
                                 max_batch_tokens=FILL_TOKENS, max_seq_len=context + PAGE,
                                 graph=False if args.no_graph else args.graph)
             view = types.SimpleNamespace(vocab_size=engine.spec.vocab_size)
+            force_what_was_asked(engine, args)
             runs = Runs(engine, view, context, args.dtype, args.samples, bracket)
             flops = (vivevik_flops(cfg, args.prefill_tokens) if label == "vivevik" else
                      ruvalorn_flops(cfg, args.prefill_tokens) if label == "ruvalorn" else

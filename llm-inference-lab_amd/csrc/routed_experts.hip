@@ -84,51 +84,75 @@ __global__ __launch_bounds__(64) void moe_select_kernel(const float* __restrict_
   }
 }
 
-// The same for a router of up to 64 outputs: a lane an output, everything in registers, no LDS
-// and no barrier.  A lane finds its place in the order (value down, index up) by reading every
-// other lane's value in turn (a read of a lane that is the same for the whole wave, which costs a
-// few clocks; a chain of lane-to-lane exchanges per chosen output would cost a hundred each).
-__device__ __forceinline__ float lane_value(float v, int lane) {
-  return __builtin_bit_cast(float, __builtin_amdgcn_readlane(__builtin_bit_cast(int, v), lane));
+// The same for a router of up to 64 outputs: a lane an output, a wave a row, no block barrier.
+// A lane finds its place in the order (value down, index up) by reading every output's value
+// from the wave's own 64 floats of LDS: reads of one address by all lanes, independent of each
+// other, so they pipeline.  (A chain of lane-to-lane exchanges per chosen output, six steps of a
+// reduction each, cost 8 to 11 us for 8 rows; reads of another lane's register in a loop over
+// the outputs were no faster.)
+__device__ __forceinline__ void wave_sync() {
+  __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
+  __builtin_amdgcn_wave_barrier();
+  __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
 }
 
-__global__ __launch_bounds__(64) void moe_select_wave_kernel(const float* __restrict__ logits,
-                                                             const float* __restrict__ correction, int outputs, int groups,
-                                                             int keep, int top, float scale, int* __restrict__ chosen,
-                                                             float* __restrict__ weights) {
-  const int row = blockIdx.x, lane = threadIdx.x;
+__device__ __forceinline__ void select_row_by_wave(const float* __restrict__ logits, const float* __restrict__ correction,
+                                                   int outputs, int groups, int keep, int top, float scale,
+                                                   int* __restrict__ chosen, float* __restrict__ weights, int row,
+                                                   int lane, float* s_wave) {
   const bool mine = lane < outputs;
   const float z = mine ? logits[(size_t)row * outputs + lane] : -INFINITY;
+  wave_sync();                                 // (the row before is read out)
+  s_wave[lane] = z;
+  wave_sync();
   float m = -INFINITY;
-  for (int j = 0; j < outputs; ++j) m = fmaxf(m, lane_value(z, j));
+  for (int j = 0; j < outputs; ++j) m = fmaxf(m, s_wave[j]);
   const float p = mine ? expf(z - m) : 0.f;
+  s_wave[WAVE + lane] = p;
+  wave_sync();
   float sum = 0.f;
-  for (int j = 0; j < outputs; ++j) sum += lane_value(p, j);         // (in the order of the outputs, on every lane)
+  for (int j = 0; j < outputs; ++j) sum += s_wave[WAVE + j];         // (in the order of the outputs, on every lane)
   const float score = p * (1.f / sum);
   float choice = mine ? score + correction[lane] : -INFINITY;
+  wave_sync();
+  s_wave[lane] = choice;
+  wave_sync();
   if (keep < groups) {
     const int per = outputs / groups, g = mine ? lane / per : groups;
     float best = -INFINITY;                    // of this lane's group
-    for (int j = 0; j < outputs; ++j) {
-      const float c = lane_value(choice, j);
-      if (j / per == g) best = fmaxf(best, c);
-    }
+    if (mine)
+      for (int i = 0; i < per; ++i) best = fmaxf(best, s_wave[g * per + i]);
+    wave_sync();
+    s_wave[WAVE + lane] = best;
+    wave_sync();
     int before = 0;                            // groups that come before this lane's
     for (int o = 0; o < groups; ++o) {
-      const float other = lane_value(best, o * per);
+      const float other = s_wave[WAVE + o * per];
       before += (other > best) || (other == best && o < g);
     }
     if (before >= keep) choice = -INFINITY;
+    wave_sync();
+    s_wave[lane] = choice;
+    wave_sync();
   }
   int place = 0;                               // outputs that come before this lane's
   for (int j = 0; j < outputs; ++j) {
-    const float c = lane_value(choice, j);
+    const float c = s_wave[j];
     place += (c > choice) || (c == choice && j < lane);
   }
   if (mine && place < top) {
     chosen[(size_t)row * top + place] = lane;
     weights[(size_t)row * top + place] = score * scale;
   }
+}
+
+__global__ __launch_bounds__(64) void moe_select_wave_kernel(const float* __restrict__ logits,
+                                                             const float* __restrict__ correction, int outputs, int groups,
+                                                             int keep, int top, float scale, int* __restrict__ chosen,
+                                                             float* __restrict__ weights) {
+  __shared__ float s_wave[2 * WAVE];
+  select_row_by_wave(logits, correction, outputs, groups, keep, top, scale, chosen, weights, blockIdx.x, threadIdx.x,
+                     s_wave);
 }
 
 extern "C" int llmlab_moe_select(const float* logits, const float* correction, int rows, int outputs, int groups,
@@ -197,17 +221,24 @@ extern "C" int llmlab_moe_add_chosen(float* resid, const void* src, int src_dtyp
 // of a product depends on that row alone.
 constexpr int PLAN_MAX_EXPERTS = 1024;
 
-__global__ __launch_bounds__(1024) void moe_plan_kernel(const int* __restrict__ chosen, int pairs, int experts, int bm,
-                                                        int capacity, int* __restrict__ place_of,
-                                                        int* __restrict__ place_row, int* __restrict__ tile_member,
-                                                        int top) {
-  __shared__ int s_count[PLAN_MAX_EXPERTS], s_start[PLAN_MAX_EXPERTS];
+__device__ __forceinline__ void plan_by_block(const int* __restrict__ chosen, int pairs, int experts, int bm, int capacity,
+                                              int* __restrict__ place_of, int* __restrict__ place_row,
+                                              int* __restrict__ tile_member, int top, int* s_count, int* s_start) {
   const int tid = threadIdx.x, nt = blockDim.x;
   for (int e = tid; e < experts; e += nt) s_count[e] = 0;
   for (int i = tid; i < capacity; i += nt) place_row[i] = -1;
   for (int t = tid; t < capacity / bm; t += nt) tile_member[t] = -1;
   __syncthreads();
-  for (int p = tid; p < pairs; p += nt) {
+  // (four pairs a load where the pairs allow it: a thread's loads are a chain of trips to memory)
+  const int quads = (((uintptr_t)chosen | (uintptr_t)place_of) % 16 == 0) ? pairs / 4 : 0;
+  for (int q = tid; q < quads; q += nt) {
+    const int4 c = ((const int4*)chosen)[q];
+    const int e4[4] = {c.x, c.y, c.z, c.w};
+#pragma unroll
+    for (int i = 0; i < 4; ++i)
+      if (e4[i] >= 0 && e4[i] < experts) atomicAdd(&s_count[e4[i]], 1);
+  }
+  for (int p = 4 * quads + tid; p < pairs; p += nt) {
     const int e = chosen[p];
     if (e >= 0 && e < experts) atomicAdd(&s_count[e], 1);
   }
@@ -226,7 +257,21 @@ __global__ __launch_bounds__(1024) void moe_plan_kernel(const int* __restrict__ 
     s_count[e] = 0;                      // from here on: places handed out
   }
   __syncthreads();
-  for (int p = tid; p < pairs; p += nt) {
+  for (int q = tid; q < quads; q += nt) {
+    const int4 c = ((const int4*)chosen)[q];
+    const int e4[4] = {c.x, c.y, c.z, c.w};
+    int place[4];
+#pragma unroll
+    for (int i = 0; i < 4; ++i) {
+      place[i] = -1;
+      if (e4[i] >= 0 && e4[i] < experts) {
+        place[i] = s_start[e4[i]] + atomicAdd(&s_count[e4[i]], 1);
+        place_row[place[i]] = (4 * q + i) / top;
+      }
+    }
+    ((int4*)place_of)[q] = make_int4(place[0], place[1], place[2], place[3]);
+  }
+  for (int p = 4 * quads + tid; p < pairs; p += nt) {
     const int e = chosen[p];
     int place = -1;
     if (e >= 0 && e < experts) {
@@ -235,6 +280,52 @@ __global__ __launch_bounds__(1024) void moe_plan_kernel(const int* __restrict__ 
     }
     place_of[p] = place;
   }
+}
+
+__global__ __launch_bounds__(1024) void moe_plan_kernel(const int* __restrict__ chosen, int pairs, int experts, int bm,
+                                                        int capacity, int* __restrict__ place_of,
+                                                        int* __restrict__ place_row, int* __restrict__ tile_member,
+                                                        int top) {
+  __shared__ int s_count[PLAN_MAX_EXPERTS], s_start[PLAN_MAX_EXPERTS];
+  plan_by_block(chosen, pairs, experts, bm, capacity, place_of, place_row, tile_member, top, s_count, s_start);
+}
+
+// Choice and sorting of a step of few rows in one launch: the waves of the one block take the rows
+// in turn, then the block sorts what they chose (their writes are the block's own: a barrier
+// makes them seen).
+__global__ __launch_bounds__(1024) void moe_select_plan_kernel(const float* __restrict__ logits,
+                                                               const float* __restrict__ correction, int rows, int outputs,
+                                                               int groups, int keep, int top, float scale,
+                                                               int* __restrict__ chosen, float* __restrict__ weights,
+                                                               int experts, int bm, int capacity, int* __restrict__ place_of,
+                                                               int* __restrict__ place_row, int* __restrict__ tile_member) {
+  __shared__ int s_count[PLAN_MAX_EXPERTS], s_start[PLAN_MAX_EXPERTS];
+  __shared__ float s_waves[16][2 * WAVE];
+  const int wave = threadIdx.x >> 6, lane = threadIdx.x & 63, waves = blockDim.x >> 6;
+  for (int row = wave; row < rows; row += waves)
+    select_row_by_wave(logits, correction, outputs, groups, keep, top, scale, chosen, weights, row, lane, s_waves[wave]);
+  __threadfence_block();
+  __syncthreads();
+  plan_by_block(chosen, rows * top, experts, bm, capacity, place_of, place_row, tile_member, top, s_count, s_start);
+}
+
+extern "C" int llmlab_moe_select_plan(const float* logits, const float* correction, int rows, int outputs, int groups,
+                                      int keep, int top, float scale, int* chosen, float* weights, int experts, int bm,
+                                      int capacity, int* place_of, int* place_row, int* tile_member, hipStream_t stream) {
+  LLMLAB_REQUIRE(rows >= 0 && outputs > 0 && outputs <= WAVE, "moe_select_plan: a router of 1 to 64 outputs, got %d",
+                 outputs);
+  LLMLAB_REQUIRE(groups > 0 && outputs % groups == 0 && keep > 0 && keep <= groups && top > 0 &&
+                     top <= keep * (outputs / groups),
+                 "moe_select_plan: %d outputs in %d groups of which %d are kept, top %d", outputs, groups, keep, top);
+  LLMLAB_REQUIRE(experts > 0 && experts <= PLAN_MAX_EXPERTS && bm > 0, "moe_select_plan: experts=%d bm=%d", experts, bm);
+  const long need = ((long)rows * top + (long)experts * (bm - 1) + bm - 1) / bm * bm;
+  LLMLAB_REQUIRE(capacity % bm == 0 && capacity >= need, "moe_select_plan: %d places for %d pairs of %d experts", capacity,
+                 rows * top, experts);
+  if (rows == 0) return 0;
+  hipLaunchKernelGGL(moe_select_plan_kernel, dim3(1), dim3(1024), 0, stream, logits, correction, rows, outputs, groups,
+                     keep, top, scale, chosen, weights, experts, bm, capacity, place_of, place_row, tile_member);
+  LLMLAB_LAUNCH_CHECK("moe_select_plan");
+  return 0;
 }
 
 extern "C" int llmlab_moe_plan(const int* chosen, int rows, int top, int experts, int bm, int capacity, int* place_of,

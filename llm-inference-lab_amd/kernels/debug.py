@@ -85,6 +85,11 @@ class DispatchRules:
     # Grouped products in tiles of 128 rows: from this many columns of a member on the tile is
     # 256 columns wide (eight waves) instead of 128.
     grouped_wide_min_columns: int = 1024
+    # Up to this many rows the router's choice and the sorting by expert are one launch of one
+    # block whose sixteen waves take a row each (8 rows of 36 outputs: 8.6 us with the host's
+    # launch against 5.8 + 5.7 in two; a wave that takes several rows one after the other pays each
+    # row's trips to memory in turn: 64 rows 28 us).
+    select_plan_max_rows: int = 16
     # ``graph="auto"`` (engine/step.py): what one call into the kernel libraries costs the
     # host that makes it through ctypes, and the rate at which a decode step streams its
     # weights and its cache.  A decode step replayed from a HIP graph costs the host

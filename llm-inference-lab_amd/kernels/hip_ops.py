@@ -1084,6 +1084,10 @@ class HipOps:
                 lib.llmlab_moe_plan.argtypes = [_c_ptr, _c_int, _c_int, _c_int, _c_int, _c_int, _c_ptr, _c_ptr, _c_ptr,
                                                 _c_ptr]
                 lib.llmlab_moe_plan.restype = _c_int
+                lib.llmlab_moe_select_plan.argtypes = [_c_ptr, _c_ptr, _c_int, _c_int, _c_int, _c_int, _c_int, _c_float,
+                                                       _c_ptr, _c_ptr, _c_int, _c_int, _c_int, _c_ptr, _c_ptr, _c_ptr,
+                                                       _c_ptr]
+                lib.llmlab_moe_select_plan.restype = _c_int
                 lib.llmlab_moe_combine.argtypes = [_c_ptr, _c_ptr, _c_ptr, _c_int, _c_ptr, _c_ptr, _c_ptr, _c_int, _c_int,
                                                    _c_int, _c_int, _c_ptr]
                 lib.llmlab_moe_combine.restype = _c_int
@@ -1123,6 +1127,38 @@ class HipOps:
         all rows with the plain 32-bit products)."""
         return dtype == torch.bfloat16 and not self.rules.experts_one_by_one
 
+    def _new_plan(self, rows: int, top: int, num_experts: int, scratch) -> "MoePlan":
+        pairs = rows * top
+        # tiles of 128 places once an expert's share of the rows fills several of them
+        bm = 128 if pairs >= 512 * num_experts else 64
+        capacity = (pairs + num_experts * (bm - 1) + bm - 1) // bm * bm
+        return MoePlan(bm, capacity, scratch("experts.place_of", (rows, top), torch.int32),
+                       scratch("experts.place_row", (capacity,), torch.int32),
+                       scratch("experts.tile_member", (capacity // bm,), torch.int32))
+
+    def moe_select_plan_takes(self, rows: int, outputs: int) -> bool:
+        """Whether choice and sorting of a step of so many rows are one launch (``moe_select_plan``)."""
+        return 0 < rows <= self.rules.select_plan_max_rows and outputs <= 64
+
+    def moe_select_plan(self, logits, correction, groups: int, groups_keep: int, scale: float, chosen, weights,
+                        num_experts: int, scratch) -> "MoePlan":
+        """``moe_select`` and ``moe_plan`` in one launch of one block, for steps of few rows."""
+        lib = self._mixer_lib("routed_experts")
+        for t, name, dt in ((logits, "router logits", torch.float32), (correction, "router correction", torch.float32),
+                            (chosen, "chosen experts", torch.int32), (weights, "expert weights", torch.float32)):
+            self._need(t, name, dt)
+        rows, outputs = logits.shape
+        top = chosen.shape[1]
+        if (correction.numel() != outputs or tuple(chosen.shape) != (rows, top) or tuple(weights.shape) != (rows, top)
+                or not self.moe_select_plan_takes(rows, outputs)):
+            raise ValueError("moe_select_plan: shapes do not fit")
+        plan = self._new_plan(rows, top, num_experts, scratch)
+        self._call(lib.llmlab_moe_select_plan, self._ptr(logits), self._ptr(correction), rows, outputs, int(groups),
+                   int(groups_keep), top, float(scale), self._ptr(chosen), self._ptr(weights), int(num_experts), plan.bm,
+                   plan.capacity, self._ptr(plan.place_of), self._ptr(plan.place_row), self._ptr(plan.tile_member),
+                   self._stream(), lib=lib)
+        return plan
+
     def moe_plan(self, chosen, num_experts: int, scratch) -> "MoePlan":
         """Sort the ``(row, choice)`` pairs of ``chosen [rows, top]`` by expert into tiles of places
         for the grouped products; choices at or beyond ``num_experts`` (outputs without tensors)
@@ -1130,13 +1166,8 @@ class HipOps:
         lib = self._mixer_lib("routed_experts")
         self._need(chosen, "chosen experts", torch.int32)
         rows, top = chosen.shape
-        pairs = rows * top
-        # tiles of 128 places once an expert's share of the rows fills several of them
-        bm = 128 if pairs >= 512 * num_experts else 64
-        capacity = (pairs + num_experts * (bm - 1) + bm - 1) // bm * bm
-        plan = MoePlan(bm, capacity, scratch("experts.place_of", (rows, top), torch.int32),
-                       scratch("experts.place_row", (capacity,), torch.int32),
-                       scratch("experts.tile_member", (capacity // bm,), torch.int32))
+        plan = self._new_plan(rows, top, num_experts, scratch)
+        bm, capacity = plan.bm, plan.capacity
         self._call(lib.llmlab_moe_plan, self._ptr(chosen), rows, top, int(num_experts), bm, capacity,
                    self._ptr(plan.place_of), self._ptr(plan.place_row), self._ptr(plan.tile_member), self._stream(),
                    lib=lib)

@@ -105,9 +105,15 @@ class RoutedExperts(FeedForward):
         ops.linear_logits(h, self.w_router, logits)
         chosen = ctx.scratch("experts.chosen", (rows, top), torch.int32)
         weights = ctx.scratch("experts.weights", (rows, top), torch.float32)
-        ops.moe_select(logits, self.correction, self.groups, self.groups_keep, self.scale, chosen, weights)
-        if self.num_experts and getattr(ops, "moe_grouped", None) is not None and ops.moe_grouped(self.dtype):
-            self._grouped(h, residual, ctx, chosen, weights)
+        grouped = self.num_experts and getattr(ops, "moe_grouped", None) is not None and ops.moe_grouped(self.dtype)
+        plan = None
+        if grouped and ops.moe_select_plan_takes(rows, self.outputs):       # few rows: choice and sorting in one launch
+            plan = ops.moe_select_plan(logits, self.correction, self.groups, self.groups_keep, self.scale, chosen,
+                                       weights, self.num_experts, ctx.scratch)
+        else:
+            ops.moe_select(logits, self.correction, self.groups, self.groups_keep, self.scale, chosen, weights)
+        if grouped:
+            self._grouped(h, residual, ctx, chosen, weights, plan)
         elif self.num_experts:
             act = ctx.scratch("experts.act", (rows, self.kernel_size), self.dtype)
             y = ctx.scratch("experts.out", (rows, self.hidden_size), torch.float32)
@@ -122,9 +128,10 @@ class RoutedExperts(FeedForward):
         if self.shared is not None:
             self.shared.forward(h, residual, ctx)
 
-    def _grouped(self, h, residual, ctx, chosen, weights):
-        ops, rows, top = self.ops, h.shape[0], self.top
-        plan = ops.moe_plan(chosen, self.num_experts, ctx.scratch)
+    def _grouped(self, h, residual, ctx, chosen, weights, plan=None):
+        ops = self.ops
+        if plan is None:
+            plan = ops.moe_plan(chosen, self.num_experts, ctx.scratch)
         act = ctx.scratch("experts.act", (plan.capacity, self.kernel_size), self.dtype)
         ops.moe_gate_up(h, self.w_gate_up, plan, act)
         y = ctx.scratch("experts.out", (plan.capacity, self.hidden_size), torch.float32)

@@ -76,3 +76,45 @@ def test_drawn_configuration(backend, seed):
             assert rms < 0.2 * size, (raw, rms)
         engine.cache.check()
         assert engine.cache.metrics()["rows_used"] == 0
+
+
+# Two configurations at the sizes of small real models (hundreds of channels, windows of hundreds
+# of positions over pages of 64, dozens of experts), with sequences that cross several windows.
+LARGER = {
+    "X": dict(architecture="Ruvalorn", vocab=701, width=384, norm=dict(eps=1e-6), loop=dict(start=0, stop=2, times=3),
+              layers=[R.attention(6, 3, 80, 0.11, size=150, rot=(40, 20000.0),
+                                  mlp=R.moe(48, 24, 6, identity=8, scale=1.5, groups=(8, 4), shared=136)),
+                      R.attention(8, 2, 64, 0.125, size=70, rot=(64, 500.0), mlp=R.dense(320)),
+                      R.attention(3, 1, 128, 0.09, size=300, rot=(32, 100.0),
+                                  mlp=R.moe(104, 10, 2, scale=2.0, groups=(2, 1)))]),
+    "Y": dict(architecture="Ruvalorn", vocab=330, width=192, norm=dict(eps=1e-5), loop=dict(start=1, stop=2, times=2),
+              layers=[R.attention(2, 2, 112, 0.1, size=257, rot=(56, 1e6), mlp=R.dense(512)),
+                      R.attention(12, 4, 32, 0.2, size=64, rot=(8, 10.0),
+                                  mlp=R.moe(32, 62, 5, identity=2, scale=3.0, groups=(16, 5), shared=64)),
+                      R.attention(4, 1, 48, 0.15, rot=(48, 10000.0), mlp=None)]),
+}
+
+
+@pytest.mark.gpu
+@pytest.mark.parametrize("name", list(LARGER))
+def test_sizes_of_small_real_models(name):
+    raw = LARGER[name]
+    cfg = H.lab.RuvalornConfig.from_dict(raw)
+    tensors = R.make_tensors(cfg, 11)
+    seqs = {f"r{i}": R.random_ids(cfg, n, 50 + i) for i, n in enumerate([420, 97, 333, 1])}
+    want = {rid: R.plain_of(cfg.to_dict(), tensors, ids) for rid, ids in seqs.items()}
+    size = max(1.0, float(torch.cat(list(want.values())).std()))
+    for dtype in ("f32", "bf16"):
+        engine = H.lab.Engine(config=cfg, tensors=tensors.items(), dtype=dtype, page_size=64, num_pages=16,
+                              max_requests=3, max_batch_tokens=512, max_seq_len=512)
+        for steps in (H.steps_prefill_then_decode(seqs, tail=40), H.steps_mixed(seqs, seed=1, max_live=3, budget=150)):
+            got = H.run_trace(engine, seqs, steps)
+            diff = torch.cat([got[rid].double() - want[rid] for rid in got])
+            assert not torch.isnan(diff).any()
+            if dtype == "f32":
+                bad = H.first_wrong(got, want, 3e-4 * size)
+                assert bad is None, f"first wrong logits at (request, position, error) = {bad}"
+            else:
+                assert float(diff.pow(2).mean().sqrt()) < 0.2 * size
+            engine.cache.check()
+            assert engine.cache.metrics()["rows_used"] == 0
