@@ -86,7 +86,7 @@ LARGER = {
                                   mlp=R.moe(48, 24, 6, identity=8, scale=1.5, groups=(8, 4), shared=136)),
                       R.attention(8, 2, 64, 0.125, size=70, rot=(64, 500.0), mlp=R.dense(320)),
                       R.attention(3, 1, 128, 0.09, size=300, rot=(32, 100.0),
-                                  mlp=R.moe(104, 10, 2, scale=2.0, groups=(2, 1)))]),
+                                  mlp=R.moe(104, 70, 3, identity=2, scale=2.0, groups=(8, 3)))]),
     "Y": dict(architecture="Ruvalorn", vocab=330, width=192, norm=dict(eps=1e-5), loop=dict(start=1, stop=2, times=2),
               layers=[R.attention(2, 2, 112, 0.1, size=257, rot=(56, 1e6), mlp=R.dense(512)),
                       R.attention(12, 4, 32, 0.2, size=64, rot=(8, 10.0),
